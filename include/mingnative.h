@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MN_VERSION 127 /* 0.1.27: parallel-mixer sequence models (section 10).  0.1.26: latent-cache sequence models (section 9).  0.1.24: mn_persist_set_status_word; mn_tp_allreduce PUSH|REDUCE above the one-shot row limit implies GATHER.  0.1.23: ABI guards mn_sizeof_* / mn_struct_layout.  0.1.20: fp8 weight mode (section 7): wfmt / row-scale fields at the END of mn_skinny_args, mn_rf_head,
+#define MN_VERSION 128 /* 0.1.28: hybrid-mixer sequence models (section 11).  0.1.27: parallel-mixer sequence models (section 10).  0.1.26: latent-cache sequence models (section 9).  0.1.24: mn_persist_set_status_word; mn_tp_allreduce PUSH|REDUCE above the one-shot row limit implies GATHER.  0.1.23: ABI guards mn_sizeof_* / mn_struct_layout.  0.1.20: fp8 weight mode (section 7): wfmt / row-scale fields at the END of mn_skinny_args, mn_rf_head,
                           mn_llm and mn_llm_tp (zero = bf16: callers of 0.1.10 that zero-fill the structs are unchanged),
                           mn_quant_fp8_rows / mn_dequant_fp8_rows / mn_stream_mfma_w8 / mn_stream_mfma_grouped_w8 */
 
@@ -948,6 +948,13 @@ MN_API int mn_window_pool_attn_blocks_ex(const float* q, int64_t ldq, const floa
                                          int one_row, int H, int G, int dim, int vdim, int t_max, int n_pool_max, int window, int pool,
                                          float out_scale, float* out, int64_t ldo, uint16_t* out16, int64_t ldo16, int nsplit, void* workspace,
                                          size_t workspace_bytes, int variant, void* stream);
+/* The same with a sink per query head (sink fp32 [H] on the device, or NULL): exp(sink[h]) joins the softmax's denominator of head h
+ * — it has no key and no value and is not scaled.  variant < 0: the kernel mn_window_pool_attn_blocks would choose. */
+MN_API int mn_window_pool_attn_blocks_sink(const float* q, int64_t ldq, const float* k_arena, const float* v_arena, const float* pk,
+                                           const float* pv, const float* sink, const int32_t* row_seq, const int32_t* row_slot,
+                                           const int32_t* blk_tab, int n_blk, int one_row, int H, int G, int dim, int vdim, int t_max,
+                                           int n_pool_max, int window, int pool, float out_scale, float* out, int64_t ldo, uint16_t* out16,
+                                           int64_t ldo16, int nsplit, void* workspace, size_t workspace_bytes, int variant, void* stream);
 /* minGRU over each sequence's rows: z = sigmoid(zx[m, c]), u = zx[m, n + c] (biases already added), candidate = u + 1/2 (u >= 0) or
  * sigmoid(u); S = (1 - z) S + z candidate from state fp32 [n_seq, n] (a row at slot 0 starts from zero), which is left at the
  * sequence's last row; out[m, c] = out_scale * S * silu(g[m, c]).  Rows of one sequence are consecutive (row_back as in 9). */
@@ -972,6 +979,9 @@ MN_API int mn_silu_mul_rows(const float* x, int64_t ldx, float* y, int64_t ldy, 
  * stride lda, weight block stride w_bs, C row stride ldc). */
 MN_API int mn_gemv_f32_indexed(const float* A, int64_t lda, int a_div, const uint16_t* W, int64_t ldw, int64_t w_bs, const int32_t* w_idx,
                                float* C, int64_t ldc, int Z, int N, int K, void* stream);
+/* The same where only indices in [0, n_idx) name a weight block: rows with any other index are left untouched */
+MN_API int mn_gemv_f32_indexed_upto(const float* A, int64_t lda, int a_div, const uint16_t* W, int64_t ldw, int64_t w_bs, const int32_t* w_idx,
+                                    int n_idx, float* C, int64_t ldc, int Z, int N, int K, void* stream);
 /* x[m] += mult * (sum_j w[m, j] y[r(m, j)] + sigmoid(sg[m * ldsg]) * shared[m]) with r(m, j) = slot_of ? slot_of[m * top + j] :
  * m * top + j; shared / sg may be NULL */
 MN_API int mn_moe_combine_residual(float* x, int64_t ldx, const float* y, int64_t ldy, const int32_t* slot_of, const float* w, int top,
@@ -1027,6 +1037,105 @@ MN_API size_t mn_pmix_workspace_bytes(const mn_pmix_model* m, int M);
 MN_API int mn_pmix_step(const mn_pmix_model* m, const mn_pmix_state* st, const float* x, int64_t ldx, int M, const int32_t* row_seq,
                         const int32_t* row_slot, const int32_t* row_back, const int32_t* blk_tab, int n_blk, int max_len, int flags,
                         float* out, float* trace, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * 11. Hybrid-mixer sequence models (0.1.28): decoder stacks whose layers choose their mixer — a causal softmax attention with grouped
+ *     key/value heads, per-head weighted RMS norm of queries and keys, a query temperature that grows with the position, and a learned
+ *     sink per head in the softmax's denominator; or a decayed linear-attention recurrence ("lightning" attention: S = decay S + k v^T,
+ *     o = S^T q on silu-activated projections, fp32 state per sequence, RMS norm over the joined heads times a sigmoid gate) — and
+ *     run mixer and feed-forward in PARALLEL on one normed input: x += mixer(h) + ff(h), h = RMS(x) w.  The feed-forward is dense
+ *     (squared relu) or a mixture of such experts whose router scores by softmax over all of its outputs, picks by score +
+ *     correction, weighs by the picked scores over their sum, and counts its last `pass` outputs as "the input itself"; an optional
+ *     shared expert is always on.  A contiguous range of layers may run several times with the same weights (each run owns its
+ *     cache or state).  Rows are fp32, weights bf16 [out, in]; the residual stream, norms, temperature, scores, softmax, router,
+ *     recurrence and its state are fp32 in both arithmetic modes (`arith` as in section 9 chooses the matrix products).
+ * ------------------------------------------------------------------------------------------ */
+/* Per row and head vector of qkv fp32 [M, (H + G) * dim + G * vdim]: q and k heads become x / sqrt(mean(x^2) + eps) * w (q_norm / k_norm
+ * bf16 [dim], shared by the heads; NULL: no weight); q is further multiplied by q_scale * (1 + temp_coef * ln(floor((pos + 1) /
+ * temp_every) + 1)) at position pos = row_slot[m] (temp_every <= 0: no temperature) and written to q_out [M, H * dim]; k and v are
+ * appended to k_arena [n_seq, t_max, G * dim], v_arena [n_seq, t_max, G * vdim] at (row_seq[m], row_slot[m]).  dim <= 512. */
+MN_API int mn_head_norm_temp_append(const float* qkv, int64_t ldqkv, int M, int H, int G, int dim, int vdim, const uint16_t* q_norm,
+                                    const uint16_t* k_norm, float eps, float q_scale, float temp_coef, int temp_every,
+                                    const int32_t* row_seq, const int32_t* row_slot, float* q_out, int64_t ldq, float* k_arena,
+                                    float* v_arena, int t_max, void* stream);
+/* Decayed linear attention over each sequence's rows.  qkv fp32 [M, 2 H dim + H vdim] = [q ; k ; v] BEFORE their silu; per head h
+ * S <- decay[h] S + k v^T, out[m, h vdim + c] = sum_i S[i, c] q[i]; state fp32 [n_seq, H, dim, vdim] (a row at slot 0 starts from
+ * zero) is left at the sequence's last row.  Rows of one sequence are consecutive (row_back as in section 9); decay: device fp32 [H].
+ * flags: MN_SEQ_ROWS_DISTINCT = every row is alone in its sequence (a decode step; row_back unused): a state column is then cut over
+ * the threads of a workgroup, so that one row's state is read and written by many workgroups at once. */
+MN_API int mn_lightning_rows(const float* qkv, int64_t ldqkv, int M, int H, int dim, int vdim, const float* decay, float* state,
+                             const int32_t* row_seq, const int32_t* row_slot, const int32_t* row_back, int flags, float* out, int64_t ldo,
+                             void* stream);
+/* The same as a chunked scan for steps of many rows (what mn_hyb_step runs above mn_lightning_chunk_rows() rows per step): chunks of
+ * rows of one sequence (chunk_tab int32 [n_chunks, 2] = (first row, rows <= mn_lightning_chunk_rows()), in row order); pass 1: every
+ * chunk's own sum of decayed k v^T; pass 2: the states at the chunks' starts, carried along each sequence; pass 3: every chunk's
+ * outputs from its start state and its own keys.  workspace from mn_lightning_scan_workspace_bytes. */
+MN_API int mn_lightning_chunk_rows(void);
+MN_API size_t mn_lightning_scan_workspace_bytes(int n_chunks, int H, int dim, int vdim);
+MN_API int mn_lightning_rows_scan(const float* qkv, int64_t ldqkv, int M, int H, int dim, int vdim, const float* decay, float* state,
+                                  const int32_t* row_seq, const int32_t* row_slot, const int32_t* row_back, const int32_t* chunk_tab,
+                                  int n_chunks, float* out, int64_t ldo, void* workspace, size_t workspace_bytes, void* stream);
+/* y = x / sqrt(mean(x^2) + eps) * w * sigmoid(g); y16: optional bf16 copy */
+MN_API int mn_rms_sigmoid_gate_rows(const float* x, int64_t ldx, const uint16_t* w, float eps, const float* g, int64_t ldg, float* y,
+                                    int64_t ldy, uint16_t* y16, int64_t ldy16, int M, int n, void* stream);
+/* y = max(x, 0)^2; y16: optional bf16 copy */
+MN_API int mn_relu2_rows(const float* x, int64_t ldx, float* y, int64_t ldy, uint16_t* y16, int64_t ldy16, int M, int n, void* stream);
+/* Router: s = softmax(logits[m, 0 .. n)); the `top` largest of s + correction (device fp32 [n] or NULL; ties: the lower index); w = their
+ * s over (the sum of their s + 1e-20).  Outputs at or past n_real name no expert ("pass the input through"): each is written as
+ * index n_real.  idx int32 [M, top], w fp32 [M, top].  n <= 512.  relu_n > 0: the same launch also writes relu_y[m, c] =
+ * max(relu_x[m, c], 0)^2 for c < relu_n (the shared expert's activation of decode rows reads the same stacked projection). */
+MN_API int mn_router_softmax_topk_rows(const float* logits, int64_t ld, int M, int n, int n_real, int top, const float* correction,
+                                       int32_t* idx, float* w, const float* relu_x, int64_t ldrx, float* relu_y, int64_t ldry, int relu_n,
+                                       void* stream);
+/* x[m] += add[m] + sum_j w[m, j] * (idx[m, j] < n_real ? y[r(m, j)] : h[m]) with r as in mn_moe_combine_residual; add may be NULL */
+MN_API int mn_moe_combine_pass_residual(float* x, int64_t ldx, const float* y, int64_t ldy, const int32_t* slot_of, const int32_t* idx,
+                                        const float* w, int top, int n_real, const float* h, int64_t ldh, const float* add, int64_t ldadd,
+                                        int M, int n, void* stream);
+
+enum { MN_HYB_ATTENTION = 0, MN_HYB_LIGHTNING = 1 };
+enum { MN_HYB_FF_NONE = 0, MN_HYB_FF_DENSE = 1, MN_HYB_FF_MOE = 2 };
+typedef struct mn_hyb_layer {
+  int32_t kind;                                    /* MN_HYB_ATTENTION | MN_HYB_LIGHTNING */
+  int32_t heads, kv_heads, dim, vdim;              /* lightning: kv_heads = heads */
+  int32_t ff_kind;                                 /* MN_HYB_FF_* */
+  int32_t ff;                                      /* dense: the feed-forward's width; moe: the shared expert's (0: none) */
+  int32_t experts, pass, top, expert_ff;           /* moe: the router has experts + pass outputs, the last `pass` stand for the input itself */
+  int32_t temp_every;                              /* attention: 0 = no query temperature */
+  float scale, temp_coef;
+  const float* sink;                               /* attention: DEVICE fp32 [heads] or NULL */
+  const float* decay;                              /* lightning: DEVICE fp32 [heads] */
+  const float* correction;                         /* moe: DEVICE fp32 [experts + pass] or NULL */
+  const uint16_t *norm1;                           /* [width] */
+  const uint16_t *q_norm, *k_norm;                 /* attention: [dim] */
+  const uint16_t *mix_norm;                        /* lightning: [heads * vdim] */
+  const uint16_t *w_in;                            /* rows [q ; k ; v ; (lightning: gate) ; up of the dense or shared expert ; router ; zero rows up to a multiple of 8] x width */
+  const uint16_t *w_out;                           /* [width, heads * vdim + ff] = [mixer o | down of the dense or shared expert] */
+  const uint16_t *w_up;                            /* moe: [experts, expert_ff, width] */
+  const uint16_t *w_down;                          /* moe: [experts, width, expert_ff] */
+} mn_hyb_layer;
+typedef struct mn_hyb_model {
+  int32_t width, n_layers, n_runs, arith;
+  float eps;
+  const mn_hyb_layer* layers;                      /* HOST array [n_layers] */
+  const int32_t* run_layer;                        /* HOST [n_runs]: the layer of every run */
+  const uint16_t* final_w;
+} mn_hyb_model;
+typedef struct mn_hyb_state {                      /* HOST arrays [n_runs] of device pointers, fp32 */
+  float* const* k;                                 /* attention runs: [n_seq, t_max, kv_heads * dim] */
+  float* const* v;                                 /* attention runs: [n_seq, t_max, kv_heads * vdim] */
+  float* const* lin;                               /* lightning runs: [n_seq, heads, dim, vdim] */
+  int32_t n_seq, t_max;
+} mn_hyb_state;
+MN_API size_t mn_sizeof_hyb_layer(void);
+MN_API size_t mn_sizeof_hyb_model(void);
+MN_API size_t mn_sizeof_hyb_state(void);
+/* One pass of the stack over M rows; rows, row arrays, blk_tab / n_blk, max_len, flags, out and trace as mn_pmix_step (trace: fp32
+ * [n_runs, M, width]).  chunk_tab / n_chunks: the rows cut into chunks of <= mn_lightning_chunk_rows() consecutive rows of one
+ * sequence (NULL / 0: the recurrences walk their rows one by one). */
+MN_API size_t mn_hyb_workspace_bytes(const mn_hyb_model* m, int M);
+MN_API int mn_hyb_step(const mn_hyb_model* m, const mn_hyb_state* st, const float* x, int64_t ldx, int M, const int32_t* row_seq,
+                       const int32_t* row_slot, const int32_t* row_back, const int32_t* blk_tab, int n_blk, const int32_t* chunk_tab,
+                       int n_chunks, int max_len, int flags, float* out, float* trace, void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

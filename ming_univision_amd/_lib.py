@@ -143,11 +143,28 @@ class PmixState(C.Structure):
                [("n_seq", C.c_int32), ("t_max", C.c_int32), ("n_pool_max", C.c_int32)]
 
 
+class HybLayer(C.Structure):
+    _fields_ = [(k, C.c_int32) for k in ("kind", "heads", "kv_heads", "dim", "vdim", "ff_kind", "ff", "experts", "n_pass", "top", "expert_ff",
+                                         "temp_every")] + \
+               [(k, C.c_float) for k in ("scale", "temp_coef")] + \
+               [(k, C.c_void_p) for k in ("sink", "decay", "correction", "norm1", "q_norm", "k_norm", "mix_norm", "w_in", "w_out", "w_up", "w_down")]
+
+
+class HybModel(C.Structure):
+    _fields_ = [("width", C.c_int32), ("n_layers", C.c_int32), ("n_runs", C.c_int32), ("arith", C.c_int32), ("eps", C.c_float),
+                ("layers", C.POINTER(HybLayer)), ("run_layer", C.POINTER(C.c_int32)), ("final_w", C.c_void_p)]
+
+
+class HybState(C.Structure):
+    _fields_ = [(k, PP) for k in ("k", "v", "lin")] + [("n_seq", C.c_int32), ("t_max", C.c_int32)]
+
+
 # (struct id of mn_struct_layout, its mn_sizeof_* export, the ctypes mirror): checked against the library at load time (`lib()`)
 STRUCTS = ((0, "mn_sizeof_skinny_args", SkinnyArgs), (1, "mn_sizeof_rf_head", RfHead), (2, "mn_sizeof_llm", Llm),
            (3, "mn_sizeof_semdec", SemDec), (4, "mn_sizeof_tp_comm", TpComm), (5, "mn_sizeof_llm_tp", LlmTp),
            (6, "mn_sizeof_seq_layer", SeqLayer), (7, "mn_sizeof_seq_model", SeqModel), (8, "mn_sizeof_seq_state", SeqState),
-           (9, "mn_sizeof_pmix_layer", PmixLayer), (10, "mn_sizeof_pmix_model", PmixModel), (11, "mn_sizeof_pmix_state", PmixState))
+           (9, "mn_sizeof_pmix_layer", PmixLayer), (10, "mn_sizeof_pmix_model", PmixModel), (11, "mn_sizeof_pmix_state", PmixState),
+           (12, "mn_sizeof_hyb_layer", HybLayer), (13, "mn_sizeof_hyb_model", HybModel), (14, "mn_sizeof_hyb_state", HybState))
 
 
 def check_struct_layouts(handle):
@@ -335,6 +352,22 @@ SYMBOLS = {
                                         _p, _sz, _p]),
     "mn_window_pool_attn_blocks_ex": (_i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _p, _i64, _p, _i64,
                                            _i, _p, _sz, _i, _p]),
+    "mn_window_pool_attn_blocks_sink": (_i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _p, _i64, _p,
+                                             _i64, _i, _p, _sz, _i, _p]),
+    "mn_gemv_f32_indexed_upto": (_i, [_p, _i64, _i, _p, _i64, _i64, _p, _i, _p, _i64, _i, _i, _i, _p]),
+    # section 11: hybrid-mixer sequence models
+    "mn_sizeof_hyb_layer": (_sz, []), "mn_sizeof_hyb_model": (_sz, []), "mn_sizeof_hyb_state": (_sz, []),
+    "mn_head_norm_temp_append": (_i, [_p, _i64, _i, _i, _i, _i, _i, _p, _p, _f, _f, _f, _i, _p, _p, _p, _i64, _p, _p, _i, _p]),
+    "mn_lightning_rows": (_i, [_p, _i64, _i, _i, _i, _i, _p, _p, _p, _p, _p, _i, _p, _i64, _p]),
+    "mn_lightning_chunk_rows": (_i, []),
+    "mn_lightning_scan_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "mn_lightning_rows_scan": (_i, [_p, _i64, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _i, _p, _i64, _p, _sz, _p]),
+    "mn_rms_sigmoid_gate_rows": (_i, [_p, _i64, _p, _f, _p, _i64, _p, _i64, _p, _i64, _i, _i, _p]),
+    "mn_relu2_rows": (_i, [_p, _i64, _p, _i64, _p, _i64, _i, _i, _p]),
+    "mn_router_softmax_topk_rows": (_i, [_p, _i64, _i, _i, _i, _i, _p, _p, _p, _p, _i64, _p, _i64, _i, _p]),
+    "mn_moe_combine_pass_residual": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _i, _i, _p, _i64, _p, _i64, _i, _i, _p]),
+    "mn_hyb_workspace_bytes": (_sz, [C.POINTER(HybModel), _i]),
+    "mn_hyb_step": (_i, [C.POINTER(HybModel), C.POINTER(HybState), _p, _i64, _i, _p, _p, _p, _p, _i, _p, _i, _i, _i, _p, _p, _p, _sz, _p]),
     "mn_semdec_step": (_i, [C.POINTER(SemDec), _p, _i, _p, _p, _p, _p, _i, _i64, _p, _p, _p, _sz, _p]),
 }
 
@@ -355,7 +388,7 @@ def lib():
         fn = getattr(handle, name)  # AttributeError if the symbol is missing
         fn.restype = res
         fn.argtypes = args
-    if handle.mn_version() < 127:
+    if handle.mn_version() < 128:
         raise RuntimeError("libmingnative.so is too old")
     check_struct_layouts(handle)
     _lib = handle

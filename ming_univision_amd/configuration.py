@@ -492,6 +492,110 @@ def sakinex_param_shapes(cfg: SakinexConfig):
     return s
 
 
+# ---- Zuzenex ---------------------------------------------------------------------------------------------------------------
+ZUZENEX_MIXERS = ("attention", "lightning")
+
+
+class ZuzenexConfig(_Config):
+    """A stack of layers that run their mixer and their feed-forward in parallel on one normed input.  `layers` is a list of
+    dicts(type, mixer, mlp):
+    type  "attention": causal softmax attention — mixer dict(heads, kv_heads, dim, vdim, scale, optional q_temp dict(coef, every)):
+                       queries and keys RMS-normed per head with a weight, the query at position p multiplied by
+                       1 + coef ln(floor((p + 1) / every) + 1), one learned sink per head in the softmax's denominator
+          "lightning": decayed linear attention — mixer dict(heads, dim, vdim, decay = one factor per head)
+    mlp   None, dict(kind="dense", ff) or dict(kind="moe", router dict(experts, top, optional identity = router outputs past the
+          experts that pass the input through), expert dict(ff), optional shared dict(ff))
+    loop  dict(start, stop, times): layers start .. stop - 1 run `times` times in a row with the same weights (every run owns its cache
+    or state).  Every size is read from here or from the tensors; nothing is assumed equal between layers."""
+    model_type = "zuzenex"
+
+    def __init__(self, width=256, vocab=1024, layers=(), norm=None, loop=None, architecture="Zuzenex", **kwargs):
+        self.architecture = architecture
+        self.width, self.vocab = int(width), int(vocab)
+        self.layers = [copy.deepcopy(dict(ly)) for ly in layers]
+        self.norm = dict(norm or {"eps": 1e-6})
+        self.loop = dict(loop) if loop else None
+        super().__init__(**kwargs)
+        self.validate()
+
+    eps = property(lambda self: float(self.norm["eps"]))
+
+    def runs(self):
+        """The layer of every run, in execution order."""
+        n = len(self.layers)
+        if not self.loop:
+            return list(range(n))
+        a, b, times = int(self.loop["start"]), int(self.loop["stop"]), int(self.loop["times"])
+        return list(range(a)) + list(range(a, b)) * times + list(range(b, n))
+
+    def validate(self):
+        if self.loop:
+            a, b, times = (int(self.loop[k]) for k in ("start", "stop", "times"))
+            if not (0 <= a <= b <= len(self.layers)) or times < 1:
+                raise ValueError(f"loop {self.loop}: 0 <= start <= stop <= {len(self.layers)} layers and times >= 1")
+        for i, ly in enumerate(self.layers):
+            if ly.get("type") not in ZUZENEX_MIXERS:
+                raise ValueError(f"layer {i}: unknown mixer type {ly.get('type')!r} (known: {ZUZENEX_MIXERS})")
+            m = ly["mixer"]
+            need = ("heads", "kv_heads", "dim", "vdim", "scale") if ly["type"] == "attention" else ("heads", "dim", "vdim", "decay")
+            for k in need:
+                if k not in m:
+                    raise ValueError(f"layer {i}: mixer lacks {k!r}")
+            if ly["type"] == "attention":
+                if int(m["heads"]) % int(m["kv_heads"]):
+                    raise ValueError(f"layer {i}: {m['heads']} query heads do not divide over {m['kv_heads']} key/value heads")
+                qt = m.get("q_temp")
+                if qt and int(qt["every"]) < 1:
+                    raise ValueError(f"layer {i}: q_temp.every must be >= 1")
+            elif len(m["decay"]) != int(m["heads"]):
+                raise ValueError(f"layer {i}: {len(m['decay'])} decay factors for {m['heads']} heads")
+            mlp = ly.get("mlp")
+            if mlp is None:
+                continue
+            if mlp.get("kind") == "dense":
+                if int(mlp["ff"]) < 1:
+                    raise ValueError(f"layer {i}: dense feed-forward needs ff >= 1")
+            elif mlp.get("kind") == "moe":
+                r = mlp["router"]
+                if int(r["experts"]) < 1 or not (1 <= int(r["top"]) <= int(r["experts"]) + int(r.get("identity") or 0)):
+                    raise ValueError(f"layer {i}: router {r}: experts >= 1 and 1 <= top <= experts + identity")
+            else:
+                raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+
+
+def zuzenex_param_shapes(cfg: ZuzenexConfig):
+    """{tensor name: shape} of a Zuzenex checkpoint (`l<i>.` per layer, `mix.` the mixer's and `mlp.` the feed-forward's tensors)."""
+    W, V = cfg.width, cfg.vocab
+    s = {"embed": (V, W)}
+    for i, ly in enumerate(cfg.layers):
+        p, m, mlp = f"l{i}.", ly["mixer"], ly.get("mlp")
+        H, d, e = int(m["heads"]), int(m["dim"]), int(m["vdim"])
+        s[p + "norm1"] = (W,)
+        if ly["type"] == "attention":
+            G = int(m["kv_heads"])
+            s[p + "mix.q"], s[p + "mix.k"], s[p + "mix.v"] = (H * d, W), (G * d, W), (G * e, W)
+            s[p + "mix.q.norm"], s[p + "mix.k.norm"], s[p + "mix.sink"] = (d,), (d,), (H,)
+        else:
+            s[p + "mix.q"], s[p + "mix.k"], s[p + "mix.v"], s[p + "mix.g"] = (H * d, W), (H * d, W), (H * e, W), (H * e, W)
+            s[p + "mix.norm"] = (H * e,)
+        s[p + "mix.o"] = (W, H * e)
+        if mlp is None:
+            continue
+        if mlp["kind"] == "dense":
+            s[p + "mlp.up"], s[p + "mlp.down"] = (int(mlp["ff"]), W), (W, int(mlp["ff"]))
+            continue
+        r = mlp["router"]
+        E, n_out, ff = int(r["experts"]), int(r["experts"]) + int(r.get("identity") or 0), int(mlp["expert"]["ff"])
+        for j in range(E):
+            s[f"{p}mlp.e{j}.up"], s[f"{p}mlp.e{j}.down"] = (ff, W), (W, ff)
+        s[p + "mlp.router"], s[p + "mlp.correction"] = (n_out, W), (n_out,)
+        if mlp.get("shared"):
+            fs = int(mlp["shared"]["ff"])
+            s[p + "mlp.shared.up"], s[p + "mlp.shared.down"] = (fs, W), (W, fs)
+    s["final.norm"], s["head"] = (W,), (V, W)
+    return s
+
+
 # ---- registry: which configuration class a config.json belongs to -------------------------------------------------------------
 def _is_pizitar(d):
     return d.get("architecture") == "Pizitar" or d.get("model_type") == "pizitar"
@@ -501,11 +605,16 @@ def _is_sakinex(d):
     return d.get("architecture") == "Sakinex" or d.get("model_type") == "sakinex"
 
 
+def _is_zuzenex(d):
+    return d.get("architecture") == "Zuzenex" or d.get("model_type") == "zuzenex"
+
+
 def _is_ming_univision(d):
     return "llm_config" in d or d.get("model_type") in ("bailingmm", "ming_univision")
 
 
-MODEL_REGISTRY = [("pizitar", _is_pizitar, PizitarConfig), ("sakinex", _is_sakinex, SakinexConfig), ("ming_univision", _is_ming_univision, MingUniVisionConfig)]
+MODEL_REGISTRY = [("pizitar", _is_pizitar, PizitarConfig), ("sakinex", _is_sakinex, SakinexConfig), ("zuzenex", _is_zuzenex, ZuzenexConfig),
+                  ("ming_univision", _is_ming_univision, MingUniVisionConfig)]
 
 
 def config_from_pretrained(path):

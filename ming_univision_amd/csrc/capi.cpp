@@ -146,13 +146,32 @@ extern "C" int mn_struct_layout(int which, size_t* offsets, int cap) {
       F(k) F(v) F(pk) F(pv) F(canon) F(conv) F(gru) F(n_seq) F(t_max) F(n_pool_max)
 #undef F
   };
-  const size_t* tab[] = {skinny, rf, llm, semdec, comm, llm_tp, seq_layer, seq_model, seq_state, pmix_layer, pmix_model, pmix_state};
+  static const size_t hyb_layer[] = {
+#define F(f) MN_OFF(mn_hyb_layer, f)
+      F(kind) F(heads) F(kv_heads) F(dim) F(vdim) F(ff_kind) F(ff) F(experts) F(pass) F(top) F(expert_ff) F(temp_every) F(scale) F(temp_coef)
+      F(sink) F(decay) F(correction) F(norm1) F(q_norm) F(k_norm) F(mix_norm) F(w_in) F(w_out) F(w_up) F(w_down)
+#undef F
+  };
+  static const size_t hyb_model[] = {
+#define F(f) MN_OFF(mn_hyb_model, f)
+      F(width) F(n_layers) F(n_runs) F(arith) F(eps) F(layers) F(run_layer) F(final_w)
+#undef F
+  };
+  static const size_t hyb_state[] = {
+#define F(f) MN_OFF(mn_hyb_state, f)
+      F(k) F(v) F(lin) F(n_seq) F(t_max)
+#undef F
+  };
+  const size_t* tab[] = {skinny, rf, llm, semdec, comm, llm_tp, seq_layer, seq_model, seq_state, pmix_layer, pmix_model, pmix_state,
+                         hyb_layer, hyb_model, hyb_state};
   const int cnt[] = {(int)(sizeof(skinny) / sizeof(size_t)), (int)(sizeof(rf) / sizeof(size_t)), (int)(sizeof(llm) / sizeof(size_t)),
                      (int)(sizeof(semdec) / sizeof(size_t)), (int)(sizeof(comm) / sizeof(size_t)), (int)(sizeof(llm_tp) / sizeof(size_t)),
                      (int)(sizeof(seq_layer) / sizeof(size_t)), (int)(sizeof(seq_model) / sizeof(size_t)),
                      (int)(sizeof(seq_state) / sizeof(size_t)), (int)(sizeof(pmix_layer) / sizeof(size_t)),
-                     (int)(sizeof(pmix_model) / sizeof(size_t)), (int)(sizeof(pmix_state) / sizeof(size_t))};
-  MN_CHECK_ARG(which >= 0 && which < 12, "mn_struct_layout: unknown struct id");
+                     (int)(sizeof(pmix_model) / sizeof(size_t)), (int)(sizeof(pmix_state) / sizeof(size_t)),
+                     (int)(sizeof(hyb_layer) / sizeof(size_t)), (int)(sizeof(hyb_model) / sizeof(size_t)),
+                     (int)(sizeof(hyb_state) / sizeof(size_t))};
+  MN_CHECK_ARG(which >= 0 && which < 15, "mn_struct_layout: unknown struct id");
   for (int i = 0; i < cnt[which] && i < cap; ++i) offsets[i] = tab[which][i];
   return cnt[which];
 }

@@ -503,7 +503,17 @@ struct AttnTArgs {
   float out_scale;
   float* out; int64_t ldo; bf16_t* out16; int64_t ldo16;
   float* part;
+  const float* sink;    // optional fp32 [H]: exp(sink[h]) joins the softmax's denominator of head h (no key, no value)
 };
+
+// 1 / (the softmax's normaliser) of a vector with running maximum m and sum l (of exp(score - m)), the head's sink included:
+// numerator and denominator are both taken relative to max(m, sink)
+__device__ __forceinline__ float softmax_inv(float m, float l, const float* sink, int h) {
+  if (!sink) return 1.0f / l;
+  const float sk = sink[h], mm = fmaxf(m, sk);
+  const float f = expf(m - mm);
+  return f / (l * f + expf(sk - mm));
+}
 
 __device__ __forceinline__ int win_t0(int pos, int window) { return window > 0 ? max(0, pos - window + 1) : 0; }
 __device__ __forceinline__ int win_nb(int pos, int window, int pool) {
@@ -671,7 +681,7 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(AttnTArgs a) {
       if (part_out) {
         part_out[2 * AQ + (int64_t)i * a.vdim + c0 + cc] = t;
       } else {
-        const float val = t / st_l[i] * a.out_scale;
+        const float val = t * softmax_inv(st_m[i], st_l[i], a.sink, h0 + i % Rc) * a.out_scale;
         const int64_t col = (int64_t)(h0 + i % Rc) * a.vdim + c0 + cc;
         const int row = r0 + i / Rc;
         if (a.out) a.out[(int64_t)row * a.ldo + col] = val;
@@ -808,7 +818,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(AttnTArgs a) {
     if (qv >= nqv) continue;
     const int row = r0 + qv / Rc;
     const int64_t col0 = (int64_t)(h0 + qv % Rc) * a.vdim;
-    const float inv = a.out_scale / lrun[i];
+    const float inv = a.out_scale * softmax_inv(mrun[i], lrun[i], a.sink, h0 + qv % Rc);
 #pragma unroll
     for (int c = 0; c < NBV; ++c) {
       const int d = 16 * (wave + 4 * c) + c16;
@@ -839,7 +849,7 @@ __global__ __launch_bounds__(256) void window_attn_merge_kernel(AttnTArgs a) {
   const float* base = a.part + ((int64_t)b * gridDim.y + gy) * a.nsplit * stride;
   // the weight of every (vector, split) once per workgroup: exp(its maximum - the overall maximum), and the vectors' normalisers
   __shared__ float wgt[AQ * 64];
-  __shared__ float Ls[AQ];
+  __shared__ float Ls[AQ], Ms[AQ];
   for (int i = tid >> 6; i < AQ; i += 4) {            // one wave per vector, one lane per split (at most 64)
     const int lane = tid & 63;
     const bool on = lane < a.nsplit;
@@ -849,7 +859,7 @@ __global__ __launch_bounds__(256) void window_attn_merge_kernel(AttnTArgs a) {
     const float w = ms == -INFINITY ? 0.f : expf(ms - mx);
     wgt[i * 64 + lane] = w;
     const float L = wave_sum(ls * w);
-    if (lane == 0) Ls[i] = L;
+    if (lane == 0) { Ls[i] = L; Ms[i] = mx; }
   }
   __syncthreads();
   for (int e = tid; e < nqv * a.vdim; e += 256) {
@@ -858,8 +868,7 @@ __global__ __launch_bounds__(256) void window_attn_merge_kernel(AttnTArgs a) {
     float t = 0.f;
 #pragma unroll 4
     for (int s = 0; s < a.nsplit; ++s) t = fmaf(src[s * stride], wgt[i * 64 + s], t);
-    const float L = Ls[i];
-    const float val = t / L * a.out_scale;
+    const float val = t * softmax_inv(Ms[i], Ls[i], a.sink, h0 + i % Rc) * a.out_scale;
     const int64_t col = (int64_t)(h0 + i % Rc) * a.vdim + c;
     const int row = r0 + i / Rc;
     if (a.out) a.out[(int64_t)row * a.ldo + col] = val;
@@ -1017,9 +1026,9 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__
 template <bool VEC>
 __global__ __launch_bounds__(256) void gemv_indexed_kernel(const float* __restrict__ A, int64_t lda, int a_div, const bf16_t* __restrict__ W,
                                                            int64_t ldw, int64_t w_bs, const int32_t* __restrict__ w_idx,
-                                                           float* __restrict__ C, int64_t ldc, int N, int K) {
+                                                           float* __restrict__ C, int64_t ldc, int N, int K, int n_idx) {
   const int z = blockIdx.y, n = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (n >= N) return;
+  if (n >= N || (unsigned)w_idx[z] >= (unsigned)n_idx) return;      // an index that names no weight block: the row is left as it is
   const float* ar = A + (int64_t)(z / a_div) * lda;
   const bf16_t* wr = W + (int64_t)w_idx[z] * w_bs + (int64_t)n * ldw;
   float acc = 0.f;
@@ -1210,6 +1219,17 @@ extern "C" int mn_window_pool_attn_blocks_ex(const float* q, int64_t ldq, const 
                                              int one_row, int H, int G, int dim, int vdim, int t_max, int n_pool_max, int window, int pool,
                                              float out_scale, float* out, int64_t ldo, uint16_t* out16, int64_t ldo16, int nsplit, void* workspace,
                                              size_t workspace_bytes, int variant, void* stream) {
+  return mn_window_pool_attn_blocks_sink(q, ldq, k_arena, v_arena, pk, pv, nullptr, row_seq, row_slot, blk_tab, n_blk, one_row, H, G, dim, vdim,
+                                         t_max, n_pool_max, window, pool, out_scale, out, ldo, out16, ldo16, nsplit, workspace, workspace_bytes,
+                                         variant, stream);
+}
+
+extern "C" int mn_window_pool_attn_blocks_sink(const float* q, int64_t ldq, const float* k_arena, const float* v_arena, const float* pk,
+                                               const float* pv, const float* sink, const int32_t* row_seq, const int32_t* row_slot,
+                                               const int32_t* blk_tab, int n_blk, int one_row, int H, int G, int dim, int vdim, int t_max,
+                                               int n_pool_max, int window, int pool, float out_scale, float* out, int64_t ldo, uint16_t* out16,
+                                               int64_t ldo16, int nsplit, void* workspace, size_t workspace_bytes, int variant, void* stream) {
+  if (variant < 0) variant = (!one_row && dim <= 256 && vdim <= 256) ? MN_WINDOW_ATTN_MFMA : MN_WINDOW_ATTN_VALU;
   MN_CHECK_ARG(q && k_arena && v_arena && row_seq && row_slot && (out || out16) && n_blk >= 1 && H >= 1 && G >= 1 && (H % G) == 0 && dim >= 1 &&
                    vdim >= 1 && vdim <= 512 && t_max >= 1 && window >= 0 && pool >= 0 && nsplit >= 1 && nsplit <= 64,
                "mn_window_pool_attn_blocks: bad args (vdim=%d: at most 512; nsplit=%d: at most 64)", vdim, nsplit);
@@ -1220,7 +1240,7 @@ extern "C" int mn_window_pool_attn_blocks_ex(const float* q, int64_t ldq, const 
   MN_CHECK_ARG(nsplit == 1 || (workspace && workspace_bytes >= mn_window_attn_workspace_bytes(n_blk, H, G, vdim, one_row, nsplit)),
                "mn_window_pool_attn_blocks: workspace too small");
   AttnTArgs a{q, ldq, k_arena, v_arena, pool ? pk : nullptr, pool ? pv : nullptr, row_seq, row_slot, one_row ? nullptr : blk_tab, H, G, dim, vdim,
-              t_max, n_pool_max, window, pool, sh.rows, sh.hpc, nsplit, out_scale, out, ldo, out16, ldo16, (float*)workspace};
+              t_max, n_pool_max, window, pool, sh.rows, sh.hpc, nsplit, out_scale, out, ldo, out16, ldo16, (float*)workspace, sink};
   MN_CHECK_ARG(variant == MN_WINDOW_ATTN_VALU || (variant == MN_WINDOW_ATTN_MFMA && !one_row && dim <= 256 && vdim <= 256),
                "mn_window_pool_attn_blocks: the matrix-core kernel takes runs of rows with dim, vdim <= 256");
   if (variant == MN_WINDOW_ATTN_MFMA) {
@@ -1323,11 +1343,17 @@ extern "C" int mn_silu_mul_rows(const float* x, int64_t ldx, float* y, int64_t l
 
 extern "C" int mn_gemv_f32_indexed(const float* A, int64_t lda, int a_div, const uint16_t* W, int64_t ldw, int64_t w_bs,
                                    const int32_t* w_idx, float* C, int64_t ldc, int Z, int N, int K, void* stream) {
-  MN_CHECK_ARG(A && W && w_idx && C && a_div >= 1 && Z >= 1 && Z <= 65535 && N >= 1 && K >= 1, "mn_gemv_f32_indexed: bad args (Z=%d)", Z);
+  return mn_gemv_f32_indexed_upto(A, lda, a_div, W, ldw, w_bs, w_idx, 0x7fffffff, C, ldc, Z, N, K, stream);
+}
+
+extern "C" int mn_gemv_f32_indexed_upto(const float* A, int64_t lda, int a_div, const uint16_t* W, int64_t ldw, int64_t w_bs,
+                                        const int32_t* w_idx, int n_idx, float* C, int64_t ldc, int Z, int N, int K, void* stream) {
+  MN_CHECK_ARG(A && W && w_idx && C && a_div >= 1 && Z >= 1 && Z <= 65535 && N >= 1 && K >= 1 && n_idx >= 1,
+               "mn_gemv_f32_indexed: bad args (Z=%d)", Z);
   const bool vec = (K % 8) == 0 && (ldw % 8) == 0 && (w_bs % 8) == 0 && (lda % 4) == 0 && (((uintptr_t)W | (uintptr_t)A) & 15) == 0;
   const dim3 grid((unsigned)mn_cdiv(N, 4), (unsigned)Z);
-  if (vec) hipLaunchKernelGGL((gemv_indexed_kernel<true>), grid, dim3(256), 0, mn_stream(stream), A, lda, a_div, W, ldw, w_bs, w_idx, C, ldc, N, K);
-  else hipLaunchKernelGGL((gemv_indexed_kernel<false>), grid, dim3(256), 0, mn_stream(stream), A, lda, a_div, W, ldw, w_bs, w_idx, C, ldc, N, K);
+  if (vec) hipLaunchKernelGGL((gemv_indexed_kernel<true>), grid, dim3(256), 0, mn_stream(stream), A, lda, a_div, W, ldw, w_bs, w_idx, C, ldc, N, K, n_idx);
+  else hipLaunchKernelGGL((gemv_indexed_kernel<false>), grid, dim3(256), 0, mn_stream(stream), A, lda, a_div, W, ldw, w_bs, w_idx, C, ldc, N, K, n_idx);
   MN_CHECK_LAUNCH("mn_gemv_f32_indexed");
   return MN_OK;
 }

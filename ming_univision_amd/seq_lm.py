@@ -1,9 +1,10 @@
 """What the decoder-only language models of this framework share: stepping rows of several cache sequences through a stack in
 passes, the vocabulary projection and the picks, a decode step captured as a HIP graph, and the lock-step generation loop.
 
-A decoder class (`pizitar.PizitarDecoder`, `sakinex.SakinexDecoder`) owns its weights, caches and states and gives
+A decoder class (`pizitar.PizitarDecoder`, `sakinex.SakinexDecoder`, `zuzenex.ZuzenexDecoder`) owns its weights, caches and states and gives
     step(x, row_seq, row_slot, row_back, row_len, blk_tab, max_len, out, trace, ws, distinct)   one pass over <= max_rows() rows
     _workspace_bytes(rows, max_len), ensure_sequences(n), release_sequences(n), n_trace (residual streams a trace holds)
+(a decoder with a `chunk_rows` attribute also gets chunk_tab = its rows cut into chunks of that many rows of one sequence)
 and inherits the rest from `SeqDecoder`; its generation entry point derives from `SeqCausalLM`.
 """
 import ctypes as C
@@ -46,13 +47,14 @@ class SeqDecoder:
             r1 = min(M, r0 + self.max_rows())
             part = [(seq, min(starts[i + 1], r1) - max(starts[i], r0), past + max(starts[i], r0) - starts[i])
                     for i, (seq, n, past) in enumerate(spans) if min(starts[i + 1], r1) > max(starts[i], r0)]
-            tabs = rows_of_spans([(int(s), int(n), int(p)) for s, n, p in part], self.block_rows)
+            tabs = rows_of_spans([(int(s), int(n), int(p)) for s, n, p in part], self.block_rows, getattr(self, "chunk_rows", 0))
             dev = {k: torch.from_numpy(v).to(self.device) for k, v in tabs.items() if k != "max_len"}
             ptr_tr = None
             if trace:
                 ptr_tr = torch.empty(self.n_trace, r1 - r0, self.cfg.width, dtype=torch.float32, device=self.device)
             self.step(x[r0:r1], dev["row_seq"], dev["row_slot"], dev["row_back"], dev["row_len"], dev["blk_tab"], tabs["max_len"],
-                      out=out[r0:r1], trace=ptr_tr, distinct=all(n == 1 for _, n, _ in part))
+                      out=out[r0:r1], trace=ptr_tr, distinct=all(n == 1 for _, n, _ in part),
+                      **({"chunk_tab": dev["chunk_tab"]} if "chunk_tab" in dev else {}))
             if trace:
                 tr[:, r0:r1] = ptr_tr
         return (out, tr) if trace else out

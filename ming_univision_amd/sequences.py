@@ -40,11 +40,12 @@ class SequenceSlots:
         return sum(self.length.values())
 
 
-def rows_of_spans(spans, block_rows):
+def rows_of_spans(spans, block_rows, chunk_rows=0):
     """spans: [(seq, n rows, past)] in row order -> dict of int32 numpy arrays: row_seq, row_slot (= position), row_back (earlier
     rows of the same sequence in this pass), row_len (= slot + 1), blk_tab [n_blk, 2] (first row, rows <= block_rows; a block never
-    crosses a span), and max_len."""
-    seqs, slots, backs, blks = [], [], [], []
+    crosses a span), and max_len.  chunk_rows > 0: also chunk_tab [n_chunks, 2], the same cut in pieces of <= chunk_rows rows (the
+    chunks of a recurrence's scan)."""
+    seqs, slots, backs, blks, chunks = [], [], [], [], []
     r0 = 0
     for seq, n, past in spans:
         seqs.append(np.full(n, seq, np.int32))
@@ -52,7 +53,13 @@ def rows_of_spans(spans, block_rows):
         backs.append(np.arange(n, dtype=np.int32))
         b0 = np.arange(0, n, block_rows, dtype=np.int32)
         blks.append(np.stack([r0 + b0, np.minimum(block_rows, n - b0)], 1))
+        if chunk_rows > 0:
+            c0 = np.arange(0, n, chunk_rows, dtype=np.int32)
+            chunks.append(np.stack([r0 + c0, np.minimum(chunk_rows, n - c0)], 1))
         r0 += n
     slot = np.concatenate(slots)
-    return dict(row_seq=np.concatenate(seqs), row_slot=slot, row_back=np.concatenate(backs), row_len=slot + 1,
-                blk_tab=np.ascontiguousarray(np.concatenate(blks).astype(np.int32)), max_len=int(slot.max()) + 1)
+    out = dict(row_seq=np.concatenate(seqs), row_slot=slot, row_back=np.concatenate(backs), row_len=slot + 1,
+               blk_tab=np.ascontiguousarray(np.concatenate(blks).astype(np.int32)), max_len=int(slot.max()) + 1)
+    if chunk_rows > 0:
+        out["chunk_tab"] = np.ascontiguousarray(np.concatenate(chunks).astype(np.int32))
+    return out
