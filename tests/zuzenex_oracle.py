@@ -75,10 +75,10 @@ def attention_mixer(h, sd, p, m, eps):
     return o.reshape(T, H * e) @ f64(sd[p + "o"]).T
 
 
-def lightning_recurrence(q, k, v, decay):
-    """q, k [T, H, d], v [T, H, e], decay [H] -> ([T, H, e], final state [H, d, e]); the state starts at zero."""
+def lightning_recurrence(q, k, v, decay, S0=None):
+    """q, k [T, H, d], v [T, H, e], decay [H] -> ([T, H, e], final state [H, d, e]); the state starts at zero (or S0)."""
     T, H, d = q.shape
-    S = torch.zeros(H, d, v.shape[2], dtype=F64)
+    S = torch.zeros(H, d, v.shape[2], dtype=F64) if S0 is None else S0.clone()
     out = torch.zeros(T, H, v.shape[2], dtype=F64)
     for t in range(T):
         S = decay[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
@@ -152,3 +152,85 @@ def forward(cfg, sd, tokens, trace=False):
         streams.append(x)
     logits = rms_norm(x, f64(sd["final.norm"]), eps) @ f64(sd["head"]).T
     return (logits, torch.stack(streams)) if trace else logits
+
+
+# ---- small models for the tests ------------------------------------------------------------------------------------------------
+def attention_layer(heads=4, kv_heads=2, dim=16, vdim=16, scale=0.25, q_temp=(0.5, 8), mlp=None):
+    m = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale)
+    if q_temp:
+        m["q_temp"] = {"coef": q_temp[0], "every": q_temp[1]}
+    return {"type": "attention", "mixer": m, "mlp": mlp}
+
+
+def lightning_layer(heads=4, dim=16, vdim=16, decay=None, mlp=None):
+    decay = decay if decay is not None else [math.exp(-0.5 / (1 + 3 * h)) for h in range(heads)]
+    return {"type": "lightning", "mixer": dict(heads=heads, dim=dim, vdim=vdim, decay=list(decay)), "mlp": mlp}
+
+
+def dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe(experts, top, ff, identity=0, shared=None):
+    m = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": ff}}
+    if identity:
+        m["router"]["identity"] = identity
+    if shared:
+        m["shared"] = {"ff": shared}
+    return m
+
+
+def small_config(layers, width=64, vocab=80, loop=None, eps=1e-5):
+    cfg = {"architecture": "Zuzenex", "width": width, "vocab": vocab, "norm": {"eps": eps}, "layers": layers}
+    if loop:
+        cfg["loop"] = dict(zip(("start", "stop", "times"), loop))
+    return cfg
+
+
+def param_shapes(cfg):
+    W, V = cfg["width"], cfg["vocab"]
+    s = {"embed": (V, W), "final.norm": (W,), "head": (V, W)}
+    for i, ly in enumerate(cfg["layers"]):
+        p, m, mlp = f"l{i}.", ly["mixer"], ly.get("mlp")
+        H, d, e = m["heads"], m["dim"], m["vdim"]
+        G = m["kv_heads"] if ly["type"] == "attention" else H
+        s.update({p + "norm1": (W,), p + "mix.q": (H * d, W), p + "mix.k": (G * d, W), p + "mix.v": (G * e, W), p + "mix.o": (W, H * e)})
+        if ly["type"] == "attention":
+            s.update({p + "mix.q.norm": (d,), p + "mix.k.norm": (d,), p + "mix.sink": (H,)})
+        else:
+            s.update({p + "mix.g": (H * e, W), p + "mix.norm": (H * e,)})
+        if mlp is None:
+            continue
+        if mlp["kind"] == "dense":
+            s.update({p + "mlp.up": (mlp["ff"], W), p + "mlp.down": (W, mlp["ff"])})
+            continue
+        r = mlp["router"]
+        n = r["experts"] + r.get("identity", 0)
+        for j in range(r["experts"]):
+            s.update({f"{p}mlp.e{j}.up": (mlp["expert"]["ff"], W), f"{p}mlp.e{j}.down": (W, mlp["expert"]["ff"])})
+        s.update({p + "mlp.router": (n, W), p + "mlp.correction": (n,)})
+        if mlp.get("shared"):
+            s.update({p + "mlp.shared.up": (mlp["shared"]["ff"], W), p + "mlp.shared.down": (W, mlp["shared"]["ff"])})
+    return s
+
+
+def random_weights(cfg, seed=0):
+    """bf16 tensors under the checkpoint's names: norm weights around 1, sinks of deviation 1, corrections large enough to change picks."""
+    g = torch.Generator().manual_seed(seed)
+    sd = {}
+    for k, shp in param_shapes(cfg).items():
+        r = torch.randn(shp, generator=g)
+        if k == "embed":
+            t = r
+        elif "norm" in k:
+            t = 1.0 + 0.1 * r
+        elif k.endswith("sink"):
+            t = r
+        elif k.endswith("correction"):
+            t = 0.05 * r
+        elif k.endswith("router"):
+            t = 2.0 * r * shp[-1] ** -0.5
+        else:
+            t = 1.3 * r * shp[-1] ** -0.5
+        sd[k] = t.to(torch.bfloat16)
+    return sd
