@@ -333,7 +333,7 @@ MN_API int mn_moe_sort_tiles(const int32_t* topk_idx, int T, int n_slot, int n_g
 /* Grouped gemm256 over that tile list (tile_rows = 128 for a hi/lo A, 256 for a plain bf16 A with a_lo_off = 0): no workgroup
  * runs for an empty tile, whatever the split of the rows over the experts.  A has a_rows_total rows.
  *   epi 0: C fp32 [*, N];  1: C bf16 [*, N];  4: W_g holds 2N rows (gate, up), C = bf16 hi rows + lo rows c_lo_off further of
- *   silu(gate) * up;  6: the same as plain bf16.   max_mtiles >= sum_g ceil(cnt[g] / tile_rows). */
+ *   silu(gate) * up;  6: the same as plain bf16;  7: C bf16 [*, N] = max(., 0)^2.   max_mtiles >= sum_g ceil(cnt[g] / tile_rows). */
 MN_API int mn_gemm256_grouped_tiles(const uint16_t* A, int64_t lda, int64_t a_lo_off, int64_t a_rows_total, const int32_t* a_rows,
                              const uint16_t* W, int64_t ldw, int64_t w_gstride, const int32_t* off, const int32_t* cnt, int n_groups,
                              const int32_t* tile_g, const int32_t* tile_m0, const int32_t* n_tiles, int max_mtiles, void* C,
@@ -1072,6 +1072,7 @@ MN_API int mn_lightning_rows(const float* qkv, int64_t ldqkv, int M, int H, int 
  * outputs from its start state and its own keys.  workspace from mn_lightning_scan_workspace_bytes. */
 MN_API int mn_lightning_chunk_rows(void);
 MN_API size_t mn_lightning_scan_workspace_bytes(int n_chunks, int H, int dim, int vdim);
+MN_API size_t mn_lightning_scan_lds_bytes(int dim, int vdim);   /* LDS a workgroup of the scan needs: the scan takes heads with at most 64 KiB */
 MN_API int mn_lightning_rows_scan(const float* qkv, int64_t ldqkv, int M, int H, int dim, int vdim, const float* decay, float* state,
                                   const int32_t* row_seq, const int32_t* row_slot, const int32_t* row_back, const int32_t* chunk_tab,
                                   int n_chunks, float* out, int64_t ldo, void* workspace, size_t workspace_bytes, void* stream);

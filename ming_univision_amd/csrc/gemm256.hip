@@ -82,7 +82,8 @@ typedef const __attribute__((address_space(1))) void glb_void;
 typedef mn_g256 G256;
 
 enum { E_F32 = MN_G256_F32, E_BF16 = MN_G256_BF16, E_BF16_GELU = MN_G256_BF16_GELU, E_F32_RESID = MN_G256_F32_RESID,
-       E_SWIGLU_SPLIT = MN_G256_SWIGLU_SPLIT, E_F32_RESID_GATE = MN_G256_F32_RESID_GATE, E_SWIGLU_BF16 = MN_G256_SWIGLU_BF16 };
+       E_SWIGLU_SPLIT = MN_G256_SWIGLU_SPLIT, E_F32_RESID_GATE = MN_G256_F32_RESID_GATE, E_SWIGLU_BF16 = MN_G256_SWIGLU_BF16,
+       E_BF16_RELU2 = MN_G256_BF16_RELU2 };
 __host__ __device__ constexpr bool epi_paired(int epi) { return epi == E_SWIGLU_SPLIT || epi == E_SWIGLU_BF16; }
 
 __device__ __forceinline__ int lds_off(int buf, int op, int half) { return ((buf * 2 + op) * 2 + half) * HALF_BYTES; }
@@ -156,8 +157,12 @@ __device__ __forceinline__ void g256_emit(const G256& p, char* Cz, int m, int n,
     f32x4* c = reinterpret_cast<f32x4*>(Cz + ((int64_t)m * p.ldc + n) * 4);
     const f32x4 g = *reinterpret_cast<const f32x4*>(p.gate + (int64_t)m * p.ldgate + n);
     *c += g * v;
-  } else if (EPI == E_BF16 || EPI == E_BF16_GELU) {
+  } else if (EPI == E_BF16 || EPI == E_BF16_GELU || EPI == E_BF16_RELU2) {
     if (EPI == E_BF16_GELU) v = f32x4{gelu_erf_bf16out(v.x), gelu_erf_bf16out(v.y), gelu_erf_bf16out(v.z), gelu_erf_bf16out(v.w)};
+    if (EPI == E_BF16_RELU2) {                         // the squared relu of a feed-forward's hidden units
+      const f32x4 r = f32x4{fmaxf(v.x, 0.f), fmaxf(v.y, 0.f), fmaxf(v.z, 0.f), fmaxf(v.w, 0.f)};
+      v = r * r;
+    }
     *reinterpret_cast<u32x2*>(Cz + ((int64_t)m * p.ldc + n) * 2) = u32x2{cvt_pk_bf16(v.x, v.y), cvt_pk_bf16(v.z, v.w)};
   } else if (EPI == E_SWIGLU_BF16) {   // y = silu(gate) * up as plain bf16 (the batched bf16 path)
     *reinterpret_cast<u32x2*>(Cz + ((int64_t)m * p.ldc + n) * 2) =
@@ -446,6 +451,7 @@ static int g256_launch(const G256& a, int epi, int ksplit, hipStream_t st) {
     case E_SWIGLU_SPLIT: G256_GO(E_SWIGLU_SPLIT); break;
     case E_F32_RESID_GATE: G256_GO(E_F32_RESID_GATE); break;
     case E_SWIGLU_BF16: G256_GO(E_SWIGLU_BF16); break;
+    case E_BF16_RELU2: G256_GO(E_BF16_RELU2); break;
     default: mn_set_error("gemm256: bad epilogue %d", epi); return MN_EINVAL;
   }
 #undef G256_GO
@@ -605,7 +611,8 @@ extern "C" int mn_gemm256_grouped_tiles(const uint16_t* A, int64_t lda, int64_t 
   const bool paired = epi == E_SWIGLU_SPLIT || epi == E_SWIGLU_BF16;
   MN_CHECK_ARG(A && W && C && off && cnt && tile_g && tile_m0 && n_tiles && n_groups >= 1 && max_mtiles >= 1 && a_lo_off >= 0 &&
                    a_rows_total >= 1, "mn_gemm256_grouped_tiles: bad args");
-  MN_CHECK_ARG(epi == E_F32 || epi == E_BF16 || epi == E_SWIGLU_SPLIT || epi == E_SWIGLU_BF16, "mn_gemm256_grouped_tiles: epi %d", epi);
+  MN_CHECK_ARG(epi == E_F32 || epi == E_BF16 || epi == E_SWIGLU_SPLIT || epi == E_SWIGLU_BF16 || epi == E_BF16_RELU2,
+               "mn_gemm256_grouped_tiles: epi %d", epi);
   MN_CHECK_ARG(N >= 4 && (N % 4) == 0 && K >= BK && (K % BK) == 0 && (lda % 8) == 0 && (ldw % 8) == 0 && (a_lo_off % 8) == 0 &&
                    (w_gstride % 8) == 0 && (((uintptr_t)A | (uintptr_t)W) & 15) == 0 && (epi != E_SWIGLU_SPLIT || c_lo_off > 0) &&
                    (a_rows_total * lda + a_lo_off) * 2 < ((int64_t)1 << 32) && (int64_t)(paired ? 2 : 1) * N * ldw * 2 < ((int64_t)1 << 32) &&

@@ -176,6 +176,9 @@ extern "C" int mn_hyb_step(const mn_hyb_model* m, const mn_hyb_state* st, const 
   hipLaunchKernelGGL(copy_rows_kernel, dim3((unsigned)mn_cdiv(W, 256), (unsigned)M), dim3(256), 0, hs, x, ldx, xr, W);
   MN_CHECK_LAUNCH("mn_hyb_step(copy)");
   const float* pend = nullptr;                      // a sublayer result that has not been added to x yet
+  // decode rows without bf16 copies: residual add + norm as one workgroup per row with the row in registers (the launch the
+  // parallel-mixer step uses for its decode rows, here without a filter)
+  const bool fuse = one_row && !want16 && W <= 8192;
   for (int ri = 0; ri < m->n_runs; ++ri) {
     const int li = m->run_layer[ri];
     MN_CHECK_ARG(li >= 0 && li < m->n_layers, "mn_hyb_step: run %d names layer %d", ri, li);
@@ -190,7 +193,8 @@ extern "C" int mn_hyb_step(const mn_hyb_model* m, const mn_hyb_state* st, const 
                  "mn_hyb_step: layer %d: bad sizes or null weights", li);
     MN_CHECK_ARG(attn ? (st->k[ri] && st->v[ri]) : st->lin[ri] != nullptr, "mn_hyb_step: run %d: null state", ri);
     // ---- the input both sublayers read, and their stacked projections ----
-    MN_TRY(mn_axpy_rms_rows(xr, W, pend, W, 1.0f, l.norm1, m->eps, hf, W, hh, W, M, W, stream));
+    if (fuse) MN_TRY(mn_axpy_rms_filter_rows(xr, W, pend, W, 1.0f, l.norm1, m->eps, nullptr, 0, nullptr, row_seq, row_slot, hf, W, M, W, stream));
+    else MN_TRY(mn_axpy_rms_rows(xr, W, pend, W, 1.0f, l.norm1, m->eps, hf, W, hh, W, M, W, stream));
     pend = nullptr;
     MN_TRY(linear(arith, M, hf, W, hh, W, l.w_in, d.n_in, W, nullptr, pin, d.n_in, gws, gwb, stream));
     // ---- mixer ----
@@ -203,7 +207,7 @@ extern "C" int mn_hyb_step(const mn_hyb_model* m, const mn_hyb_state* st, const 
                                              l.heads, l.kv_heads, l.dim, l.vdim, st->t_max, 1, 0, 0, 1.0f, cat, d.n_cat, cath, d.n_cat, ns, aws,
                                              p.attn_ws, -1, stream));
     } else {
-      const size_t lds3 = ((size_t)mn_lightning_chunk_rows() * (2 * l.dim + l.vdim + mn_lightning_chunk_rows() + 1)) * sizeof(float);
+      const size_t lds3 = mn_lightning_scan_lds_bytes(l.dim, l.vdim);
       const bool scan = !one_row && chunk_tab && n_chunks >= 1 && M >= 2 * mn_lightning_chunk_rows() && lds3 <= 64 * 1024 &&
                         mn_lightning_scan_workspace_bytes(n_chunks, l.heads, l.dim, l.vdim) <= scan_cap;
       if (scan)
@@ -239,8 +243,7 @@ extern "C" int mn_hyb_step(const mn_hyb_model* m, const mn_hyb_state* st, const 
         const int max_mtiles = Z / 256 + E;
         MN_TRY(mn_ep_dispatch(tidx, M, top, E + 1, 0, E, counts, offsets, perm, slot_of, 256, tile_g, tile_m0, n_tiles, stream));
         MN_TRY(mn_gemm256_grouped_tiles(h16, W, 0, M, perm, l.w_up, W, (int64_t)eff * W, offsets, counts, E, tile_g, tile_m0, n_tiles, max_mtiles,
-                                        gu, eff, 0, eff, W, 0, stream));
-        MN_TRY(mn_relu2_rows(gu, eff, nullptr, 0, eah, eff, Z, eff, stream));
+                                        eah, eff, 0, eff, W, 7, stream));          // the squared relu in the epilogue
         MN_TRY(mn_gemm256_grouped_tiles(eah, eff, 0, Z, nullptr, l.w_down, eff, (int64_t)W * eff, offsets, counts, E, tile_g, tile_m0, n_tiles,
                                         max_mtiles, ye, W, 0, W, eff, 0, stream));
         so = slot_of;
@@ -268,7 +271,8 @@ extern "C" int mn_hyb_step(const mn_hyb_model* m, const mn_hyb_state* st, const 
       MN_CHECK_LAUNCH("mn_hyb_step(trace)");
     }
   }
-  MN_TRY(mn_axpy_rms_rows(xr, W, pend, W, 1.0f, m->final_w, m->eps, out, W, nullptr, 0, M, W, stream));
+  if (fuse) MN_TRY(mn_axpy_rms_filter_rows(xr, W, pend, W, 1.0f, m->final_w, m->eps, nullptr, 0, nullptr, row_seq, row_slot, out, W, M, W, stream));
+  else MN_TRY(mn_axpy_rms_rows(xr, W, pend, W, 1.0f, m->final_w, m->eps, out, W, nullptr, 0, M, W, stream));
 #undef MN_TRY
   return MN_OK;
 }

@@ -192,6 +192,19 @@ struct LightScanArgs {
 };
 __device__ __forceinline__ float powi32(float lam, float loglam, int p) { return p == 0 ? 1.0f : (lam > 0.f ? expf((float)p * loglam) : 0.f); }
 
+// CV value columns per thread (4: 16-byte loads of the values and the carried state; needs vdim % 4 == 0), the rows of the result
+// split over the thread groups that share a column group
+template <int CV>
+__device__ __forceinline__ void ld_cols(const float* p, float (&v)[CV]) {
+  if constexpr (CV == 4) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  } else {
+    v[0] = *p;
+  }
+}
+
+template <int CV>
 __global__ __launch_bounds__(256) void light_scan_kv_kernel(LightScanArgs s) {
   extern __shared__ float lds[];             // k [LCH][dim] (decayed), v [LCH][vdim]
   const LightArgs& a = s.b;
@@ -210,25 +223,34 @@ __global__ __launch_bounds__(256) void light_scan_kv_kernel(LightScanArgs s) {
   }
   __syncthreads();
   float* dst = s.ws + ((int64_t)ch * a.H + h) * d * e;
-  for (int c0 = 0; c0 < e; c0 += 256) {
-    const int cw = min(256, e - c0), nsub = 256 / cw, c = tid % cw, sub = tid / cw;
+  constexpr int R = 8;
+  const int ncg = e / CV;
+  for (int g0 = 0; g0 < ncg; g0 += 256) {
+    const int cw = min(256, ncg - g0), nsub = 256 / cw, c = CV * (g0 + tid % cw), sub = tid / cw;
     if (sub >= nsub) continue;
-    for (int ib = 0; ib < d; ib += 16 * nsub) {
-      float acc[16];
+    for (int ib = 0; ib < d; ib += R * nsub) {
+      float acc[R][CV];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int q = 0; q < CV; ++q) acc[r][q] = 0.f;
       for (int j = 0; j < n; ++j) {
-        const float vv = vl[j * e + c0 + c];
+        float vv[CV];
+        ld_cols<CV>(vl + j * e + c, vv);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
+        for (int r = 0; r < R; ++r) {
           const int i = ib + sub + r * nsub;
-          acc[r] = fmaf(kl[j * d + (i < d ? i : 0)], vv, acc[r]);
+          const float kk = kl[j * d + (i < d ? i : 0)];
+#pragma unroll
+          for (int q = 0; q < CV; ++q) acc[r][q] = fmaf(kk, vv[q], acc[r][q]);
         }
       }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
+      for (int r = 0; r < R; ++r) {
         const int i = ib + sub + r * nsub;
-        if (i < d) dst[(int64_t)i * e + c0 + c] = acc[r];
+        if (i >= d) continue;
+#pragma unroll
+        for (int q = 0; q < CV; ++q) dst[(int64_t)i * e + c + q] = acc[r][q];
       }
     }
   }
@@ -253,21 +275,22 @@ __global__ __launch_bounds__(256) void light_scan_carry_kernel(LightScanArgs s) 
   *sp = S;
 }
 
+template <int CV>
 __global__ __launch_bounds__(256) void light_scan_out_kernel(LightScanArgs s) {
-  extern __shared__ float lds[];             // q [LCH][dim], k [LCH][dim], v [LCH][vdim], P [LCH][LCH + 1]
+  extern __shared__ float lds[];             // q [LCH][dim + 1], k [LCH][dim + 1], v [LCH][vdim], P [LCH][LCH + 1]
   const LightArgs& a = s.b;
-  const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, d = a.dim, e = a.vdim;
+  const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, d = a.dim, e = a.vdim, dp = d + 1;   // odd row stride: the score loop walks rows
   const int r0 = s.chunk_tab[2 * ch], n = s.chunk_tab[2 * ch + 1];
   float* ql = lds;
-  float* kl = ql + LCH * d;
-  float* vl = kl + LCH * d;
+  float* kl = ql + LCH * dp;
+  float* vl = kl + LCH * dp + (4 - (2 * LCH * dp) % 4) % 4;      // 16-byte aligned rows of values
   float* P = vl + LCH * e;
   const float lam = a.decay[h], ll = lam > 0.f ? logf(lam) : 0.f;
   for (int x = tid; x < n * d; x += 256) {
     const int j = x / d, i = x - j * d;
     const float* row = a.qkv + (int64_t)(r0 + j) * a.ldqkv + (int64_t)h * d + i;
-    ql[x] = silu32(row[0]);
-    kl[x] = silu32(row[(int64_t)a.H * d]);
+    ql[j * dp + i] = silu32(row[0]);
+    kl[j * dp + i] = silu32(row[(int64_t)a.H * d]);
   }
   for (int x = tid; x < n * e; x += 256) {
     const int j = x / e, c = x - j * e;
@@ -278,42 +301,67 @@ __global__ __launch_bounds__(256) void light_scan_out_kernel(LightScanArgs s) {
     const int i = x / n, j = x - i * n;
     float t = 0.f;
     if (j <= i) {
-      for (int u = 0; u < d; ++u) t = fmaf(ql[i * d + u], kl[j * d + u], t);
-      t *= powi32(lam, ll, i - j);
+      float t2 = 0.f;
+      int u = 0;
+      for (; u + 1 < d; u += 2) {
+        t = fmaf(ql[i * dp + u], kl[j * dp + u], t);
+        t2 = fmaf(ql[i * dp + u + 1], kl[j * dp + u + 1], t2);
+      }
+      if (u < d) t = fmaf(ql[i * dp + u], kl[j * dp + u], t);
+      t = (t + t2) * powi32(lam, ll, i - j);
     }
     P[i * (LCH + 1) + j] = t;
   }
   __syncthreads();
   const float* S0 = s.ws + ((int64_t)ch * a.H + h) * d * e;
-  for (int c0 = 0; c0 < e; c0 += 256) {
-    const int cw = min(256, e - c0), nsub = 256 / cw, c = tid % cw, sub = tid / cw;
+  constexpr int R = 4;
+  const int ncg = e / CV;
+  for (int g0 = 0; g0 < ncg; g0 += 256) {
+    const int cw = min(256, ncg - g0), nsub = 256 / cw, c = CV * (g0 + tid % cw), sub = tid / cw;
     if (sub >= nsub) continue;
-    for (int ib = 0; ib < n; ib += 16 * nsub) {
-      float acc[16];
+    for (int ib = 0; ib < n; ib += R * nsub) {
+      float acc[R][CV];
+      int qrow[R];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-      for (int u = 0; u < d; ++u) {                    // the part that comes from the chunk's start state
-        const float sv = S0[(int64_t)u * e + c0 + c];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int i = ib + sub + r * nsub;
-          acc[r] = fmaf(ql[(i < n ? i : 0) * d + u], sv, acc[r]);
-        }
-      }
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] *= powi32(lam, ll, ib + sub + r * nsub + 1);
-      for (int j = 0; j < n; ++j) {                    // the chunk's own keys
-        const float vv = vl[j * e + c0 + c];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int i = ib + sub + r * nsub;
-          acc[r] = fmaf(P[(i < n ? i : 0) * (LCH + 1) + j], vv, acc[r]);
-        }
-      }
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
+      for (int r = 0; r < R; ++r) {
         const int i = ib + sub + r * nsub;
-        if (i < n) a.out[(int64_t)(r0 + i) * a.ldo + (int64_t)h * e + c0 + c] = acc[r];
+        qrow[r] = (i < n ? i : 0) * dp;
+#pragma unroll
+        for (int q = 0; q < CV; ++q) acc[r][q] = 0.f;
+      }
+      for (int u = 0; u < d; ++u) {                    // the part that comes from the chunk's start state
+        float sv[CV];
+        ld_cols<CV>(S0 + (int64_t)u * e + c, sv);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const float qq = ql[qrow[r] + u];
+#pragma unroll
+          for (int q = 0; q < CV; ++q) acc[r][q] = fmaf(qq, sv[q], acc[r][q]);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const float f = powi32(lam, ll, ib + sub + r * nsub + 1);
+#pragma unroll
+        for (int q = 0; q < CV; ++q) acc[r][q] *= f;
+      }
+      for (int j = 0; j < n; ++j) {                    // the chunk's own keys
+        float vv[CV];
+        ld_cols<CV>(vl + j * e + c, vv);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const int i = ib + sub + r * nsub;
+          const float pp = P[(i < n ? i : 0) * (LCH + 1) + j];
+#pragma unroll
+          for (int q = 0; q < CV; ++q) acc[r][q] = fmaf(pp, vv[q], acc[r][q]);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int i = ib + sub + r * nsub;
+        if (i >= n) continue;
+#pragma unroll
+        for (int q = 0; q < CV; ++q) a.out[(int64_t)(r0 + i) * a.ldo + (int64_t)h * e + c + q] = acc[r][q];
       }
     }
   }
@@ -489,6 +537,11 @@ extern "C" int mn_lightning_rows(const float* qkv, int64_t ldqkv, int M, int H, 
 
 extern "C" int mn_lightning_chunk_rows(void) { return LCH; }
 
+// LDS of the scan's output pass: q and k rows of dim + 1 floats, value rows, the chunk's decayed scores
+extern "C" size_t mn_lightning_scan_lds_bytes(int dim, int vdim) {
+  return ((size_t)LCH * (2 * (dim + 1) + vdim) + 4 + (size_t)LCH * (LCH + 1)) * sizeof(float);
+}
+
 extern "C" size_t mn_lightning_scan_workspace_bytes(int n_chunks, int H, int dim, int vdim) {
   if (n_chunks < 1 || H < 1 || dim < 1 || vdim < 1) return 0;
   return (size_t)n_chunks * H * dim * vdim * sizeof(float);
@@ -500,15 +553,19 @@ extern "C" int mn_lightning_rows_scan(const float* qkv, int64_t ldqkv, int M, in
   MN_CHECK_ARG(qkv && decay && state && row_seq && row_slot && row_back && chunk_tab && out && workspace && M >= 1 && H >= 1 && H <= 65535 &&
                    dim >= 1 && vdim >= 1 && n_chunks >= 1 && n_chunks <= 65535, "mn_lightning_rows_scan: bad args");
   MN_CHECK_ARG(workspace_bytes >= mn_lightning_scan_workspace_bytes(n_chunks, H, dim, vdim), "mn_lightning_rows_scan: workspace too small");
-  const size_t lds3 = ((size_t)LCH * (2 * dim + vdim) + LCH * (LCH + 1)) * sizeof(float);
+  const size_t lds3 = mn_lightning_scan_lds_bytes(dim, vdim);
   MN_CHECK_ARG(lds3 <= 64 * 1024, "mn_lightning_rows_scan: heads of %d + %d values do not fit (use mn_lightning_rows)", dim, vdim);
   LightScanArgs s{LightArgs{qkv, ldqkv, H, dim, vdim, decay, state, row_seq, row_slot, row_back, out, ldo, M}, chunk_tab, n_chunks, (float*)workspace};
   hipStream_t st = mn_stream(stream);
-  hipLaunchKernelGGL(light_scan_kv_kernel, dim3((unsigned)n_chunks, (unsigned)H), dim3(256), (size_t)LCH * (dim + vdim) * sizeof(float), st, s);
+  // four value columns per thread where rows of values and of the state are 16-byte aligned
+  const bool v4 = (vdim % 4) == 0 && (((uintptr_t)workspace) & 15) == 0;
+  if (v4) hipLaunchKernelGGL((light_scan_kv_kernel<4>), dim3((unsigned)n_chunks, (unsigned)H), dim3(256), (size_t)LCH * (dim + vdim) * sizeof(float), st, s);
+  else hipLaunchKernelGGL((light_scan_kv_kernel<1>), dim3((unsigned)n_chunks, (unsigned)H), dim3(256), (size_t)LCH * (dim + vdim) * sizeof(float), st, s);
   MN_CHECK_LAUNCH("mn_lightning_rows_scan(sums)");
   hipLaunchKernelGGL(light_scan_carry_kernel, dim3((unsigned)mn_cdiv((int64_t)dim * vdim, 256), (unsigned)H, (unsigned)n_chunks), dim3(256), 0, st, s);
   MN_CHECK_LAUNCH("mn_lightning_rows_scan(carry)");
-  hipLaunchKernelGGL(light_scan_out_kernel, dim3((unsigned)n_chunks, (unsigned)H), dim3(256), lds3, st, s);
+  if (v4) hipLaunchKernelGGL((light_scan_out_kernel<4>), dim3((unsigned)n_chunks, (unsigned)H), dim3(256), lds3, st, s);
+  else hipLaunchKernelGGL((light_scan_out_kernel<1>), dim3((unsigned)n_chunks, (unsigned)H), dim3(256), lds3, st, s);
   MN_CHECK_LAUNCH("mn_lightning_rows_scan(outputs)");
   return MN_OK;
 }

@@ -1,5 +1,5 @@
-"""Prefill / decode throughput of the Pizitar or the Sakinex decoder beside the Bailing-MoE decoder at equal size
-(`bench.py --lm-compare [--lm-model sakinex]`).
+"""Prefill / decode throughput of the Pizitar, the Sakinex or the Zuzenex decoder beside the Bailing-MoE decoder at equal size
+(`bench.py --lm-compare [--lm-model sakinex | zuzenex]`).
 
 Random weights at sizes that resemble real layers.  "Equal size": same width, depth and head count, 128-wide heads on both, and a
 feed-forward whose ACTIVE hidden width matches (the MoE runs 8 experts, top-2, of half the dense hidden width each).  Both run
@@ -15,6 +15,13 @@ no repeated layers.  Its attention reads at most window + length / pool keys per
   decode   bytes of the visible keys and values (token arenas + block-mean arenas) per step / HBM peak
   prefill  multiply-adds of the visible score / value products on the fp32 FMA peak (the kernel's arithmetic)
 and the recurrence alone on the bytes it reads and writes.
+
+Zuzenex at "equal size": same width, depth, query / key-value head counts and 128-wide heads, layers attention - lightning - lightning -
+attention, 8 experts top-2 plus one pass-through output and one shared expert (its experts have two matrices where the SwiGLU experts
+have three, so they are 1.5 times as wide: the same parameters per expert).  Its attention sees every earlier token, like the other
+decoder's, and is priced the same way — on the fp32 matrix-core peak for prompts (its scores and weights are 32-bit) and on the cache
+bytes for decode rows; the recurrence alone is priced on its multiply-adds (prompts: the chunked scan) and on the state bytes it reads
+and writes (decode rows).
 """
 import time
 
@@ -213,6 +220,101 @@ def run_sakinex(s, T, batches, n_dec):
     return out
 
 
+def zuzenex_config(s):
+    from .configuration import ZuzenexConfig
+    H = s["heads"]
+    mlp = dict(kind="moe", router=dict(experts=8, top=2, identity=1), expert=dict(ff=s["ff"] * 3 // 4), shared=dict(ff=s["ff"] * 3 // 4))
+    att = dict(type="attention", mixer=dict(heads=H, kv_heads=H // 4, dim=128, vdim=128, scale=128 ** -0.5, q_temp=dict(coef=0.1, every=1024)), mlp=mlp)
+    lin = dict(type="lightning", mixer=dict(heads=H, dim=128, vdim=128, decay=[1.0 - 2.0 ** (-5 - 4 * h / H) for h in range(H)]), mlp=mlp)
+    order = [att, lin, lin, att]
+    return ZuzenexConfig(width=s["width"], vocab=s["vocab"], layers=[order[i % 4] for i in range(s["layers"])], norm=dict(eps=1e-6))
+
+
+def run_zuzenex(s, T, batches, n_dec):
+    from ._lib import check, current_stream, lib, ptr
+    from .sequences import rows_of_spans
+    from .zuzenex import ZuzenexDecoder
+    dev = "cuda"
+    cfg = zuzenex_config(s)
+    dec = ZuzenexDecoder.synthetic(cfg, dev, t_max=T + n_dec + 8, n_seq=max(batches), arith="bf16")
+    ids = torch.randint(0, s["vocab"], (T,), device=dev)
+    x = dec.embed(ids)
+    out = {"prefill_tokens_per_s": T / _time(lambda: dec.forward_spans(x, [(0, T, 0)]), 3)}
+    for B in batches:
+        for run in dec.state_t:                              # every sequence continues the prompt of sequence 0
+            for t in run.values():
+                if t is not None and B > 1:
+                    t[1:B].copy_(t[0:1].expand_as(t[1:B]))
+        row_seq = torch.arange(B, dtype=torch.int32, device=dev)
+        back, blk = dec.decode_tables(B)
+        xb = dec.embed(torch.randint(0, s["vocab"], (B,), device=dev))
+
+        def loop():
+            slot = torch.full((B,), T, dtype=torch.int32, device=dev)
+            ln = slot + 1
+            for i in range(n_dec):
+                dec.step(xb, row_seq, slot, back, ln, blk, T + i + 1, distinct=True)
+                check(lib().mn_rows_advance(ptr(slot), ptr(ln), None, B, 1, current_stream()), "mn_rows_advance")
+        out[f"decode_b{B}_tokens_per_s"] = B * n_dec / _time(loop, 2, 1)
+        slot_g = torch.full((B,), T, dtype=torch.int32, device=dev)
+        ln_g = slot_g + 1
+        graph = dec.decode_graph(row_seq, slot_g, ln_g)
+
+        def loop_graph():
+            slot_g.fill_(T)
+            ln_g.fill_(T + 1)
+            for i in range(n_dec):
+                graph.run(xb, T + i + 1)
+        out[f"decode_b{B}_graph_tokens_per_s"] = B * n_dec / _time(loop_graph, 2, 1)
+    # the attention kernel alone, on the first run's arenas (an attention layer)
+    H, G, d = s["heads"], s["heads"] // 4, 128
+    st = dec.state_t[0]
+    RB = lib().mn_window_attn_block_rows()
+    tabs = {k: torch.from_numpy(v).to(dev) for k, v in rows_of_spans([(0, T, 0)], RB, dec.chunk_rows).items() if k != "max_len"}
+    q = torch.randn(T, H * d, device=dev) * 0.05
+    att = torch.empty(T, H * d, device=dev)
+    sink = torch.zeros(H, device=dev)
+    aws = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+
+    def attn(M, rs, rp, one_row):
+        n_blk = M if one_row else tabs["blk_tab"].shape[0]
+        ns = lib().mn_window_attn_splits(n_blk, H, G, one_row, T)
+        check(lib().mn_window_pool_attn_blocks_sink(ptr(q), H * d, ptr(st["k"]), ptr(st["v"]), None, None, ptr(sink), ptr(rs), ptr(rp),
+                                                    None if one_row else ptr(tabs["blk_tab"]), n_blk, one_row, H, G, d, d, dec.t_max, 1, 0, 0, 1.0,
+                                                    ptr(att), H * d, None, 0, ns, ptr(aws), aws.numel(), -1, current_stream()),
+              "mn_window_pool_attn_blocks_sink")
+        return ns
+    t = _time(lambda: attn(T, tabs["row_seq"], tabs["row_slot"], 0), 5)
+    flops = 2 * 2 * H * d * T * (T + 1) / 2
+    out["attn_prefill"] = dict(us=t * 1e6, tflops=flops / t / 1e12, of_peak=flops / t / 1e12 / FMA_F32_TFLOPS, peak="fp32 MFMA")
+    for B in batches:
+        row_seq = torch.arange(B, dtype=torch.int32, device=dev)
+        slot = torch.full((B,), T - 1, dtype=torch.int32, device=dev)
+        t = _time(lambda: attn(B, row_seq, slot, 1), 20)
+        byts = B * T * G * 2 * d * 4
+        out[f"attn_decode_b{B}"] = dict(us=t * 1e6, gbs=byts / t / 1e9, of_peak=byts / t / 1e9 / HBM_GBS, key_splits=attn(B, row_seq, slot, 1))
+    # the recurrence alone, on the second run's state (a lightning layer)
+    lin = dec.state_t[1]["lin"]
+    decay = torch.full((H,), 0.99, device=dev)
+    qkv, o = torch.randn(T, 3 * H * d, device=dev), torch.empty(T, H * d, device=dev)
+    n_ch = tabs["chunk_tab"].shape[0]
+    sws = torch.empty(lib().mn_lightning_scan_workspace_bytes(n_ch, H, d, d), dtype=torch.uint8, device=dev)
+    t = _time(lambda: check(lib().mn_lightning_rows_scan(ptr(qkv), 3 * H * d, T, H, d, d, ptr(decay), ptr(lin), ptr(tabs["row_seq"]), ptr(tabs["row_slot"]),
+                                                         ptr(tabs["row_back"]), ptr(tabs["chunk_tab"]), n_ch, ptr(o), H * d, ptr(sws), sws.numel(),
+                                                         current_stream()), "mn_lightning_rows_scan"), 5)
+    C = dec.chunk_rows
+    flops = 2 * T * H * (2 * d * d + C * 2 * d)             # per token and head: its k v^T, q against the carried state, the chunk's own scores and values
+    out["lightning_prefill"] = dict(us=t * 1e6, tflops=flops / t / 1e12, of_peak=flops / t / 1e12 / FMA_F32_TFLOPS, peak="fp32 FMA")
+    for B in batches:
+        row_seq = torch.arange(B, dtype=torch.int32, device=dev)
+        slot = torch.full((B,), T - 1, dtype=torch.int32, device=dev)
+        t = _time(lambda: check(lib().mn_lightning_rows(ptr(qkv), 3 * H * d, B, H, d, d, ptr(decay), ptr(lin), ptr(row_seq), ptr(slot), None, 1, ptr(o),
+                                                        H * d, current_stream()), "mn_lightning_rows"), 20)
+        byts = B * H * d * d * 4 * 2
+        out[f"lightning_decode_b{B}"] = dict(us=t * 1e6, gbs=byts / t / 1e9, of_peak=byts / t / 1e9 / HBM_GBS)
+    return out
+
+
 def run_bailing(s, T, batches, n_dec, shared=0):
     from . import ops
     from ._lib import check, current_stream, lib, ptr
@@ -262,10 +364,12 @@ def compare(sizes=("w1024", "w2048"), prompt=2048, batches=(1, 32), n_dec=32, mo
     for name in sizes:
         s = SIZES[name]
         torch.cuda.empty_cache()
-        if model == "sakinex":
+        if model == "zuzenex":
+            res[name] = dict(size=s, prompt=prompt, zuzenex=run_zuzenex(s, prompt, batches, n_dec))
+        elif model == "sakinex":
             res[name] = dict(size=s, prompt=prompt, sakinex=run_sakinex(s, prompt, batches, n_dec))
         else:
             res[name] = dict(size=s, prompt=prompt, pizitar=run_pizitar(s, prompt, batches, n_dec))
         torch.cuda.empty_cache()
-        res[name]["bailing_moe"] = run_bailing(s, prompt, batches, n_dec, shared=1 if model == "sakinex" else 0)
+        res[name]["bailing_moe"] = run_bailing(s, prompt, batches, n_dec, shared=1 if model in ("sakinex", "zuzenex") else 0)
     return res

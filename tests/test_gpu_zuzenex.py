@@ -248,7 +248,7 @@ def test_lightning_recurrence_rows_steps_and_scan(H, d, e):
     ref, fin = _light_ref(qkv[:, :C_], H, d, e, decay, spans, {s: O.f64(stale[s]) for s in range(n_seq)})
     chunk = L.mn_lightning_chunk_rows()
     r = _rows(spans, chunk_rows=chunk)
-    lds_ok = (chunk * (2 * d + e + chunk + 1)) * 4 <= 64 * 1024
+    lds_ok = L.mn_lightning_scan_lds_bytes(d, e) <= 64 * 1024
     for mode in ("rows", "scan"):
         if mode == "scan" and not lds_ok:
             continue
