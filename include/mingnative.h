@@ -1073,6 +1073,13 @@ MN_API int mn_lightning_rows(const float* qkv, int64_t ldqkv, int M, int H, int 
 MN_API int mn_lightning_chunk_rows(void);
 MN_API size_t mn_lightning_scan_workspace_bytes(int n_chunks, int H, int dim, int vdim);
 MN_API size_t mn_lightning_scan_lds_bytes(int dim, int vdim);   /* LDS a workgroup of the scan needs: the scan takes heads with at most 64 KiB */
+/* The same with the output pass named: MN_LIGHTNING_SCAN_MFMA (what mn_lightning_rows_scan runs when its tiles fit 64 KiB of LDS) =
+ * scores, carried-state and value products on the fp32 matrix cores (v_mfma_f32_16x16x4_f32: fp32 operands and accumulation);
+ * MN_LIGHTNING_SCAN_VALU = the fp32 FMA pass (the plain kernel the other is checked against). */
+enum { MN_LIGHTNING_SCAN_MFMA = 0, MN_LIGHTNING_SCAN_VALU = 1 };
+MN_API int mn_lightning_rows_scan_ex(const float* qkv, int64_t ldqkv, int M, int H, int dim, int vdim, const float* decay, float* state,
+                                     const int32_t* row_seq, const int32_t* row_slot, const int32_t* row_back, const int32_t* chunk_tab,
+                                     int n_chunks, float* out, int64_t ldo, void* workspace, size_t workspace_bytes, int variant, void* stream);
 MN_API int mn_lightning_rows_scan(const float* qkv, int64_t ldqkv, int M, int H, int dim, int vdim, const float* decay, float* state,
                                   const int32_t* row_seq, const int32_t* row_slot, const int32_t* row_back, const int32_t* chunk_tab,
                                   int n_chunks, float* out, int64_t ldo, void* workspace, size_t workspace_bytes, void* stream);

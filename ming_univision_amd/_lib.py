@@ -363,6 +363,7 @@ SYMBOLS = {
     "mn_lightning_scan_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "mn_lightning_scan_lds_bytes": (_sz, [_i, _i]),
     "mn_lightning_rows_scan": (_i, [_p, _i64, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _i, _p, _i64, _p, _sz, _p]),
+    "mn_lightning_rows_scan_ex": (_i, [_p, _i64, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _i, _p, _i64, _p, _sz, _i, _p]),
     "mn_rms_sigmoid_gate_rows": (_i, [_p, _i64, _p, _f, _p, _i64, _p, _i64, _p, _i64, _i, _i, _p]),
     "mn_relu2_rows": (_i, [_p, _i64, _p, _i64, _p, _i64, _i, _i, _p]),
     "mn_router_softmax_topk_rows": (_i, [_p, _i64, _i, _i, _i, _i, _p, _p, _p, _p, _i64, _p, _i64, _i, _p]),

@@ -3,7 +3,7 @@
 // attention) with its fp32 state, the RMS-norm x sigmoid-gate of its joined heads, the squared-relu activation, a router that scores
 // by softmax over every output, picks by score + correction and passes some picks through, and the expert combine that knows them.
 // Rows are fp32, weights bf16; everything here is fp32 arithmetic.
-#include "common.h"
+#include "mfma_f32_tiles.h"
 
 namespace {
 
@@ -367,6 +367,113 @@ __global__ __launch_bounds__(256) void light_scan_out_kernel(LightScanArgs s) {
   }
 }
 
+// Pass 3 on the fp32 matrix cores (v_mfma_f32_16x16x4_f32: fp32 operands and accumulation; operand layouts in mfma_f32_tiles.h).  A
+// workgroup of 4 waves owns one (chunk, head): q, k (rows of ldq floats) and v (rows of ldv floats) of the chunk's <= 32 rows are staged
+// activated and zero padded; waves 0 .. 2 multiply the three 16 x 16 score tiles on or below the diagonal and park them, decayed and
+// masked, in LDS; then wave w owns the 16-column tiles w, w + 4, .. of the result, both row tiles at once: Q S0 with the carried state
+// read straight from the workspace (8 loads in flight), times lam^(i + 1) by rows, plus P V.
+__global__ __launch_bounds__(256) void light_scan_out_mfma_kernel(LightScanArgs s, int ldq, int ldv) {
+  extern __shared__ float lds[];             // q [32][ldq], k [32][ldq], v [32][ldv], P [32][36]
+  constexpr int LDP = 36;
+  const LightArgs& a = s.b;
+  const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, d = a.dim, e = a.vdim;
+  const int r0 = s.chunk_tab[2 * ch], n = s.chunk_tab[2 * ch + 1];
+  const int wave = tid >> 6, lane = tid & 63, c16 = lane & 15, g4 = lane >> 4;
+  float* ql = lds;
+  float* kl = ql + LCH * ldq;
+  float* vl = kl + LCH * ldq;
+  float* P = vl + LCH * ldv;
+  const float lam = a.decay[h], ll = lam > 0.f ? logf(lam) : 0.f;
+  for (int x = tid; x < LCH * ldq; x += 256) {
+    const int j = x / ldq, i = x - j * ldq;
+    float qv = 0.f, kv = 0.f;
+    if (j < n && i < d) {
+      const float* row = a.qkv + (int64_t)(r0 + j) * a.ldqkv + (int64_t)h * d + i;
+      qv = silu32(row[0]);
+      kv = silu32(row[(int64_t)a.H * d]);
+    }
+    ql[x] = qv;
+    kl[x] = kv;
+  }
+  for (int x = tid; x < LCH * ldv; x += 256) {
+    const int j = x / ldv, c = x - j * ldv;
+    vl[x] = (j < n && c < e) ? silu32(a.qkv[(int64_t)(r0 + j) * a.ldqkv + (int64_t)2 * a.H * d + (int64_t)h * e + c]) : 0.f;
+  }
+  __syncthreads();
+  const int ksteps = (d + 3) / 4;            // ldq >= 4 ksteps, the padding is zero
+  if (wave < 3) {                            // score tiles (0, 0), (1, 0), (1, 1)
+    const int ti = wave == 0 ? 0 : 1, tj = wave == 2 ? 1 : 0;
+    f32x4 sc = f32x4{0.f, 0.f, 0.f, 0.f}, sc2 = f32x4{0.f, 0.f, 0.f, 0.f};
+    const float* ap = ql + (16 * ti + c16) * ldq + g4;
+    const float* bp = kl + (16 * tj + c16) * ldq + g4;
+    int it = 0;
+    for (; it + 1 < ksteps; it += 2) {
+      sc = __builtin_amdgcn_mfma_f32_16x16x4f32(ap[4 * it], bp[4 * it], sc, 0, 0, 0);
+      sc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(ap[4 * it + 4], bp[4 * it + 4], sc2, 0, 0, 0);
+    }
+    if (it < ksteps) sc = __builtin_amdgcn_mfma_f32_16x16x4f32(ap[4 * it], bp[4 * it], sc, 0, 0, 0);
+    sc += sc2;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 16 * ti + 4 * g4 + i, col = 16 * tj + c16;
+      P[row * LDP + col] = col <= row ? sc[i] * powi32(lam, ll, row - col) : 0.f;
+    }
+  } else {                                   // the tile above the diagonal
+    for (int x = lane; x < 256; x += 64) P[(x >> 4) * LDP + 16 + (x & 15)] = 0.f;
+  }
+  __syncthreads();
+  const float* S0 = s.ws + ((int64_t)ch * a.H + h) * d * e;
+  float rowf[2][4];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) rowf[t][i] = powi32(lam, ll, 16 * t + 4 * g4 + i + 1);
+  const int ntile = (e + 15) / 16;
+  for (int ct = wave; ct < ntile; ct += 4) {
+    const int col = 16 * ct + c16;
+    const bool col_ok = col < e;
+    const float* sp = S0 + (col_ok ? col : 0);
+    f32x4 acc0 = f32x4{0.f, 0.f, 0.f, 0.f}, acc1 = f32x4{0.f, 0.f, 0.f, 0.f};
+    const float* a0 = ql + c16 * ldq + g4;
+    const float* a1 = ql + (16 + c16) * ldq + g4;
+    for (int it0 = 0; it0 < ksteps; it0 += 8) {
+      float b[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int k = 4 * (it0 + u) + g4;
+        const float t = sp[(int64_t)(k < d ? k : 0) * e];
+        b[u] = (col_ok && k < d) ? t : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (it0 + u < ksteps) {
+          acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[4 * (it0 + u)], b[u], acc0, 0, 0, 0);
+          acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[4 * (it0 + u)], b[u], acc1, 0, 0, 0);
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { acc0[i] *= rowf[0][i]; acc1[i] *= rowf[1][i]; }
+    const float* p0 = P + c16 * LDP + g4;
+    const float* p1 = P + (16 + c16) * LDP + g4;
+    const float* vb = vl + g4 * ldv + 16 * ct + c16;
+#pragma unroll
+    for (int it = 0; it < LCH / 4; ++it) {
+      const float bv = vb[4 * it * ldv];
+      if (it < 4) acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(p0[4 * it], bv, acc0, 0, 0, 0);      // row tile 0 sees keys 0 .. 15 only
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(p1[4 * it], bv, acc1, 0, 0, 0);
+    }
+    if (col_ok) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int ra = 4 * g4 + i, rb = 16 + ra;
+        if (ra < n) a.out[(int64_t)(r0 + ra) * a.ldo + (int64_t)h * e + col] = acc0[i];
+        if (rb < n) a.out[(int64_t)(r0 + rb) * a.ldo + (int64_t)h * e + col] = acc1[i];
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------------------------------
 // one workgroup per row: y = x / sqrt(mean(x^2) + eps) * w * sigmoid(g)
 __global__ __launch_bounds__(256) void rms_sigmoid_gate_kernel(const float* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ w, float eps,
@@ -547,12 +654,28 @@ extern "C" size_t mn_lightning_scan_workspace_bytes(int n_chunks, int H, int dim
   return (size_t)n_chunks * H * dim * vdim * sizeof(float);
 }
 
+namespace {
+// row strides of the matrix-core pass: q / k rows = 4 mod 32 floats, v rows = 16 mod 32 — the operand reads of a wave then fall two to a bank
+inline int scan_ldq(int dim) { const int p = (dim + 3) / 4 * 4; return p + ((p % 32) == 0 ? 4 : ((36 - p % 32) % 32)); }
+inline int scan_ldv(int vdim) { const int p = (vdim + 15) / 16 * 16; return p + ((p % 32) == 0 ? 16 : 0); }
+inline size_t scan_mfma_lds(int dim, int vdim) { return ((size_t)LCH * (2 * scan_ldq(dim) + scan_ldv(vdim)) + LCH * 36) * sizeof(float); }
+}  // namespace
+
 extern "C" int mn_lightning_rows_scan(const float* qkv, int64_t ldqkv, int M, int H, int dim, int vdim, const float* decay, float* state,
                                       const int32_t* row_seq, const int32_t* row_slot, const int32_t* row_back, const int32_t* chunk_tab,
                                       int n_chunks, float* out, int64_t ldo, void* workspace, size_t workspace_bytes, void* stream) {
+  return mn_lightning_rows_scan_ex(qkv, ldqkv, M, H, dim, vdim, decay, state, row_seq, row_slot, row_back, chunk_tab, n_chunks, out, ldo, workspace,
+                                   workspace_bytes, scan_mfma_lds(dim, vdim) <= 64 * 1024 ? MN_LIGHTNING_SCAN_MFMA : MN_LIGHTNING_SCAN_VALU, stream);
+}
+
+extern "C" int mn_lightning_rows_scan_ex(const float* qkv, int64_t ldqkv, int M, int H, int dim, int vdim, const float* decay, float* state,
+                                         const int32_t* row_seq, const int32_t* row_slot, const int32_t* row_back, const int32_t* chunk_tab,
+                                         int n_chunks, float* out, int64_t ldo, void* workspace, size_t workspace_bytes, int variant,
+                                         void* stream) {
   MN_CHECK_ARG(qkv && decay && state && row_seq && row_slot && row_back && chunk_tab && out && workspace && M >= 1 && H >= 1 && H <= 65535 &&
                    dim >= 1 && vdim >= 1 && n_chunks >= 1 && n_chunks <= 65535, "mn_lightning_rows_scan: bad args");
   MN_CHECK_ARG(workspace_bytes >= mn_lightning_scan_workspace_bytes(n_chunks, H, dim, vdim), "mn_lightning_rows_scan: workspace too small");
+  MN_CHECK_ARG(variant == MN_LIGHTNING_SCAN_MFMA || variant == MN_LIGHTNING_SCAN_VALU, "mn_lightning_rows_scan: unknown variant %d", variant);
   const size_t lds3 = mn_lightning_scan_lds_bytes(dim, vdim);
   MN_CHECK_ARG(lds3 <= 64 * 1024, "mn_lightning_rows_scan: heads of %d + %d values do not fit (use mn_lightning_rows)", dim, vdim);
   LightScanArgs s{LightArgs{qkv, ldqkv, H, dim, vdim, decay, state, row_seq, row_slot, row_back, out, ldo, M}, chunk_tab, n_chunks, (float*)workspace};
@@ -564,7 +687,11 @@ extern "C" int mn_lightning_rows_scan(const float* qkv, int64_t ldqkv, int M, in
   MN_CHECK_LAUNCH("mn_lightning_rows_scan(sums)");
   hipLaunchKernelGGL(light_scan_carry_kernel, dim3((unsigned)mn_cdiv((int64_t)dim * vdim, 256), (unsigned)H, (unsigned)n_chunks), dim3(256), 0, st, s);
   MN_CHECK_LAUNCH("mn_lightning_rows_scan(carry)");
-  if (v4) hipLaunchKernelGGL((light_scan_out_kernel<4>), dim3((unsigned)n_chunks, (unsigned)H), dim3(256), lds3, st, s);
+  if (variant == MN_LIGHTNING_SCAN_MFMA) {
+    MN_CHECK_ARG(scan_mfma_lds(dim, vdim) <= 64 * 1024, "mn_lightning_rows_scan: heads of %d + %d values do not fit the matrix-core pass", dim, vdim);
+    hipLaunchKernelGGL(light_scan_out_mfma_kernel, dim3((unsigned)n_chunks, (unsigned)H), dim3(256), scan_mfma_lds(dim, vdim), st, s, scan_ldq(dim),
+                       scan_ldv(vdim));
+  } else if (v4) hipLaunchKernelGGL((light_scan_out_kernel<4>), dim3((unsigned)n_chunks, (unsigned)H), dim3(256), lds3, st, s);
   else hipLaunchKernelGGL((light_scan_out_kernel<1>), dim3((unsigned)n_chunks, (unsigned)H), dim3(256), lds3, st, s);
   MN_CHECK_LAUNCH("mn_lightning_rows_scan(outputs)");
   return MN_OK;

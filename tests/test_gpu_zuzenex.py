@@ -249,8 +249,8 @@ def test_lightning_recurrence_rows_steps_and_scan(H, d, e):
     chunk = L.mn_lightning_chunk_rows()
     r = _rows(spans, chunk_rows=chunk)
     lds_ok = L.mn_lightning_scan_lds_bytes(d, e) <= 64 * 1024
-    for mode in ("rows", "scan"):
-        if mode == "scan" and not lds_ok:
+    for mode in ("rows", "scan", "scan_valu"):               # "scan": the matrix-core output pass where its tiles fit
+        if mode != "rows" and not lds_ok:
             continue
         state, out = stale.clone().cuda(), torch.zeros(M, H * e, device="cuda")
         if mode == "rows":
@@ -259,8 +259,12 @@ def test_lightning_recurrence_rows_steps_and_scan(H, d, e):
         else:
             n_ch = r["chunk_tab"].shape[0]
             ws = torch.empty(L.mn_lightning_scan_workspace_bytes(n_ch, H, d, e), dtype=torch.uint8, device="cuda")
-            check(L.mn_lightning_rows_scan(ptr(D(qkv)), C_ + 1, M, H, d, e, ptr(D(decay)), ptr(state), ptr(r["row_seq"]), ptr(r["row_slot"]),
-                                           ptr(r["row_back"]), ptr(r["chunk_tab"]), n_ch, ptr(out), H * e, ptr(ws), ws.numel(), stream()))
+            if mode == "scan":
+                check(L.mn_lightning_rows_scan(ptr(D(qkv)), C_ + 1, M, H, d, e, ptr(D(decay)), ptr(state), ptr(r["row_seq"]), ptr(r["row_slot"]),
+                                               ptr(r["row_back"]), ptr(r["chunk_tab"]), n_ch, ptr(out), H * e, ptr(ws), ws.numel(), stream()))
+            else:
+                check(L.mn_lightning_rows_scan_ex(ptr(D(qkv)), C_ + 1, M, H, d, e, ptr(D(decay)), ptr(state), ptr(r["row_seq"]), ptr(r["row_slot"]),
+                                                  ptr(r["row_back"]), ptr(r["chunk_tab"]), n_ch, ptr(out), H * e, ptr(ws), ws.numel(), 1, stream()))
         assert err(out, ref) < 2e-5, mode
         for s, S in fin.items():
             assert err(state[s], S) < 2e-5, (mode, s)
