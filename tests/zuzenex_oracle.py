@@ -155,7 +155,7 @@ def forward(cfg, sd, tokens, trace=False):
 
 
 # ---- small models for the tests ------------------------------------------------------------------------------------------------
-def attention_layer(heads=4, kv_heads=2, dim=16, vdim=16, scale=0.25, q_temp=(0.5, 8), mlp=None):
+def attention_layer(heads=4, kv_heads=2, dim=16, vdim=16, scale=0.25, q_temp=(0.4, 8), mlp=None):
     m = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale)
     if q_temp:
         m["q_temp"] = {"coef": q_temp[0], "every": q_temp[1]}
@@ -163,7 +163,7 @@ def attention_layer(heads=4, kv_heads=2, dim=16, vdim=16, scale=0.25, q_temp=(0.
 
 
 def lightning_layer(heads=4, dim=16, vdim=16, decay=None, mlp=None):
-    decay = decay if decay is not None else [math.exp(-0.5 / (1 + 3 * h)) for h in range(heads)]
+    decay = decay if decay is not None else [1.0 - 0.45 / (1 + 2 * h) for h in range(heads)]
     return {"type": "lightning", "mixer": dict(heads=heads, dim=dim, vdim=vdim, decay=list(decay)), "mlp": mlp}
 
 
