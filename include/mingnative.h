@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define MN_VERSION 128 /* 0.1.28: hybrid-mixer sequence models (section 11).  0.1.27: parallel-mixer sequence models (section 10).  0.1.26: latent-cache sequence models (section 9).  0.1.24: mn_persist_set_status_word; mn_tp_allreduce PUSH|REDUCE above the one-shot row limit implies GATHER.  0.1.23: ABI guards mn_sizeof_* / mn_struct_layout.  0.1.20: fp8 weight mode (section 7): wfmt / row-scale fields at the END of mn_skinny_args, mn_rf_head,
+#define MN_VERSION 129 /* 0.1.29: post-norm mixed-mixer sequence models (section 12).  0.1.28: hybrid-mixer sequence models (section 11).  0.1.27: parallel-mixer sequence models (section 10).  0.1.26: latent-cache sequence models (section 9).  0.1.24: mn_persist_set_status_word; mn_tp_allreduce PUSH|REDUCE above the one-shot row limit implies GATHER.  0.1.23: ABI guards mn_sizeof_* / mn_struct_layout.  0.1.20: fp8 weight mode (section 7): wfmt / row-scale fields at the END of mn_skinny_args, mn_rf_head,
                           mn_llm and mn_llm_tp (zero = bf16: callers of 0.1.10 that zero-fill the structs are unchanged),
                           mn_quant_fp8_rows / mn_dequant_fp8_rows / mn_stream_mfma_w8 / mn_stream_mfma_grouped_w8 */
 
@@ -1144,6 +1144,135 @@ MN_API size_t mn_hyb_workspace_bytes(const mn_hyb_model* m, int M);
 MN_API int mn_hyb_step(const mn_hyb_model* m, const mn_hyb_state* st, const float* x, int64_t ldx, int M, const int32_t* row_seq,
                        const int32_t* row_slot, const int32_t* row_back, const int32_t* blk_tab, int n_blk, const int32_t* chunk_tab,
                        int n_chunks, int max_len, int flags, float* out, float* trace, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The block attention of section 10 with a sink per head (or NULL), a soft cap of the scores (softcap > 0: every score s becomes
+ * softcap * tanh(s / softcap) before the softmax; 0: none) and explicit row strides of the two arenas (ldk, ldv in floats; 0 = G * dim,
+ * G * vdim): the value arena may be a view into the key arena — latent attention reads keys [latent ; rotated part] and values
+ * [latent] from one arena with ldv = ldk.  A stride under heads of a multiple of 4 values must be a multiple of 4 itself. */
+MN_API int mn_window_pool_attn_blocks_cap(const float* q, int64_t ldq, const float* k_arena, int64_t ldk, const float* v_arena, int64_t ldv,
+                                          const float* pk, const float* pv, const float* sink, float softcap, const int32_t* row_seq,
+                                          const int32_t* row_slot, const int32_t* blk_tab, int n_blk, int one_row, int H, int G, int dim,
+                                          int vdim, int t_max, int n_pool_max, int window, int pool, float out_scale, float* out, int64_t ldo,
+                                          uint16_t* out16, int64_t ldo16, int nsplit, void* workspace, size_t workspace_bytes, int variant,
+                                          void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * 12. Post-norm mixed-mixer sequence models (0.1.29): decoder stacks whose sublayers read the residual stream as it is and whose
+ *     RESULTS are RMS-normed before they are added: x += w1 rms(mixer(x)), x += w2 rms(ff(x)), and optionally a per-layer token
+ *     input x += ws rms(P (gelu(G x) * e)), e a slice of a second embedding row of the token.  The mixer is chosen per layer:
+ *     softmax attention (grouped heads, biases, RMS norm over the whole q and k projections, rotary pairs with optional
+ *     long-context frequency scaling, soft-capped scores, sliding window, a sigmoid gate per head), latent attention (one normed
+ *     latent and one rotated key part per token are cached; keys and values of every head are linear maps of the latent), or the
+ *     gated delta rule (short causal filters and silu on q / k / v, unit-length q and k, a write strength and a decay per head
+ *     and token, fp32 state per sequence).  The feed-forward is W_down (gelu(W_gate x) * W_up x), gelu in its tanh form.
+ *     Rows are fp32, weights bf16 [out, in]; the residual stream, norms, angles, scores, softmax, gates, decays and the recurrent
+ *     state are fp32 in both arithmetic modes (`arith` as in section 9 chooses the matrix products).
+ * ------------------------------------------------------------------------------------------ */
+/* Rotary frequencies base^(-2i / dims), i < dims / 2, rescaled by wavelength when factor > 0: a wavelength below original / high keeps
+ * its frequency f, one above original / low gets f / factor, between them (1 - s) f / factor + s f with
+ * s = (original / wavelength - low) / (high - low).  HOST output freq [dims / 2], computed in double. */
+MN_API int mn_rotary_frequencies_scaled_host(int dims, double base, double factor, double low, double high, double original, float* freq);
+/* x += y / sqrt(mean(y^2) + eps) * w; x16: optional bf16 copy of the new x */
+MN_API int mn_rms_scale_add_rows(float* x, int64_t ldx, const float* y, int64_t ldy, const uint16_t* w, float eps, uint16_t* x16,
+                                 int64_t ldx16, int M, int n, void* stream);
+/* y[m, c] = gelu_tanh(a[m, c]) * b[m, c], or with b NULL times table[idx[m] * ldt + c] (bf16 table rows chosen per row; point
+ * `table` at the first column of the slice).  y (fp32) and y16 (bf16) are both optional outputs. */
+MN_API int mn_gelu_mul_rows(const float* a, int64_t lda, const float* b, int64_t ldb, const uint16_t* table, int64_t ldt,
+                            const int32_t* idx, float* y, int64_t ldy, uint16_t* y16, int64_t ldy16, int M, int n, void* stream);
+/* Per row of qkv fp32 [M, H dim + G dim + G vdim]: q and k are divided by the root mean square of their WHOLE projection (all heads
+ * at once) and multiplied by q_norm bf16 [H dim] / k_norm bf16 [G dim] (NULL: neither), then the first rot_dims values of every
+ * head turn by position * freq[i] (freq device fp32 [rot_dims / 2]; interleaved 1: pairs (2i, 2i + 1), 0: pairs (i, i + rot_dims / 2));
+ * q * q_scale goes to q_out [M, H dim], k and v are appended at (row_seq[m], row_slot[m]) of k_arena [n_seq, t_max, ldk] and
+ * v_arena [n_seq, t_max, ldv]. */
+MN_API int mn_proj_norm_rope_append(const float* qkv, int64_t ldqkv, int M, int H, int G, int dim, int vdim, const uint16_t* q_norm,
+                                    const uint16_t* k_norm, float eps, int rot_dims, int interleaved, const float* freq, float q_scale,
+                                    const int32_t* row_seq, const int32_t* row_slot, float* q_out, int64_t ldq, float* k_arena, int64_t ldk,
+                                    float* v_arena, int64_t ldv, int t_max, void* stream);
+/* Per row of qd fp32 [M, H (dim + rot) + rank + rot] = [queries head by head as (dim plain, rot rotated) ; down projection]:
+ * arena[seq, slot, 0 .. rank) = RMS norm of the down projection's first rank values times c_norm; arena[seq, slot, rank .. rank + rot)
+ * = its last rot values rotated; q_out[m, h (rank + rot) + rank + d] = q_scale * the rotated part of head h (the first `rank`
+ * columns of every head are left for the caller's absorbed product).  Rotation as in mn_proj_norm_rope_append on the first
+ * rot_dims <= rot values. */
+MN_API int mn_latent_rope_append(const float* qd, int64_t ld, int M, int H, int dim, int rot, int rank, const uint16_t* c_norm, float eps,
+                                 int rot_dims, int interleaved, const float* freq, float q_scale, const int32_t* row_seq,
+                                 const int32_t* row_slot, float* q_out, int64_t ldq, float* arena, int64_t lda, int t_max, void* stream);
+/* x[m, h vdim + c] *= sigmoid(g[m, h]); x16: optional bf16 copy */
+MN_API int mn_head_sigmoid_gate_rows(float* x, int64_t ldx, const float* g, int64_t ldg, uint16_t* x16, int64_t ldx16, int M, int H,
+                                     int vdim, void* stream);
+/* Gated delta rule, preparation.  proj fp32 [M, ld]: raw channels [q: G dim ; k: G dim ; v: H vdim] from column 0, the write-strength
+ * logits [H] from off_b and the decay logits [H] from off_a.  Every channel goes through its causal filter w_conv bf16 [channels, taps]
+ * (last tap = the current row; earlier inputs from the rows before it in this call, then from state fp32 [n_seq, taps - 1, channels]
+ * as mn_tap_filter_rows reads it — mn_tap_state_update moves it on afterwards) and silu; q and k heads become x / sqrt(sum(x^2) +
+ * unit_eps), q also times q_scale.  qkv fp32 [M, channels]; bd fp32 [M, 2 H] = [sigmoid(b) ; exp(-exp(a_log) softplus(a + dt_bias))]. */
+MN_API int mn_delta_prep_rows(const float* proj, int64_t ld, int M, int H, int G, int dim, int vdim, int off_b, int off_a,
+                              const uint16_t* w_conv, int taps, const float* state, const float* a_log, const float* dt_bias,
+                              float unit_eps, float q_scale, const int32_t* row_seq, const int32_t* row_slot, const int32_t* row_back,
+                              float* qkv, int64_t ldo, float* bd, int64_t ldbd, void* stream);
+/* Gated delta rule over each sequence's rows, per head h (q / k head h / (H / G)) with beta and g of the row:
+ * S <- g S; u = beta (v - S^T k); S <- S + k u^T; out[m, h vdim + c] = (S^T q)[c].  state fp32 [n_seq, H, dim, vdim] (a row at slot 0
+ * starts from zero) is left at the sequence's last row.  Rows of one sequence are consecutive (row_back as in section 9).
+ * flags: MN_SEQ_ROWS_DISTINCT = every row is alone in its sequence (a decode step).  dim <= 512. */
+MN_API int mn_gated_delta_rows(const float* qkv, int64_t ld, const float* bd, int64_t ldbd, int M, int H, int G, int dim, int vdim,
+                               float* state, const int32_t* row_seq, const int32_t* row_slot, const int32_t* row_back, int flags,
+                               float* out, int64_t ldo, void* stream);
+/* y[m, h vdim + c] = x / sqrt(mean over the head's vdim values of x^2 + eps) * w[c] * silu(g[m, h vdim + c]); y16: optional bf16 copy */
+MN_API int mn_head_rms_silu_gate_rows(const float* x, int64_t ldx, const uint16_t* w, float eps, const float* g, int64_t ldg, float* y,
+                                      int64_t ldy, uint16_t* y16, int64_t ldy16, int M, int H, int vdim, void* stream);
+
+enum { MN_PN_ATTENTION = 0, MN_PN_LATENT = 1, MN_PN_DELTA = 2 };
+typedef struct mn_pn_layer {
+  int32_t kind;                                    /* MN_PN_* */
+  int32_t heads, kv_heads, dim, vdim;              /* latent: kv_heads unused; dim = the plain part of a query / key head */
+  int32_t rot, kv_rank;                            /* latent: rotated part of a head, latent size */
+  int32_t rot_dims, rot_interleaved;               /* attention / latent: values of a head (of its rotated part) that turn; 0: none */
+  int32_t window;                                  /* attention / latent: 0 = every earlier token */
+  int32_t conv;                                    /* delta: taps of the q / k / v filters */
+  int32_t ff;                                      /* 0: no feed-forward */
+  int32_t side;                                    /* values of the per-layer token input, 0: none */
+  int32_t has_gate;                                /* attention: 1 = a sigmoid gate per head follows v in the stack */
+  float scale, softcap;                            /* softcap 0: none */
+  float unit_eps;                                  /* delta: inside the root of the unit norms */
+  const float* rot_freq;                           /* DEVICE fp32 [rot_dims / 2] */
+  const float *a_log, *dt_bias;                    /* delta: DEVICE fp32 [heads] */
+  const uint16_t *norm1, *norm2, *side_norm;       /* [width] */
+  const uint16_t *w_in, *b_in;                     /* attention [q ; k ; v ; gate], latent [q ; down], delta [q ; k ; v ; b ; a ; g]; zero rows up to a multiple of 8; bias or NULL */
+  const uint16_t *q_norm, *k_norm;                 /* attention: [heads dim], [kv_heads dim] or NULL; latent: k_norm = the latent's norm [kv_rank] */
+  const uint16_t *w_conv;                          /* delta: [2 kv_heads dim + heads vdim, conv] */
+  const uint16_t *mix_norm;                        /* delta: [vdim] */
+  const uint16_t *w_ukT;                           /* latent: [heads, kv_rank, dim] */
+  const uint16_t *w_uv;                            /* latent: [heads vdim, kv_rank] */
+  const uint16_t *w_o, *b_o;                       /* [width, heads vdim], bias or NULL */
+  const uint16_t *w_gate_up;                       /* [2 ff, width] = [gate ; up] */
+  const uint16_t *w_down;                          /* [width, ff] */
+  const uint16_t *w_side_gate;                     /* [side rounded up to a multiple of 8, width] */
+  const uint16_t *w_side_proj;                     /* [width, side] */
+  const uint16_t *side_table;                      /* the layer's first column of the token table */
+} mn_pn_layer;
+typedef struct mn_pn_model {
+  int32_t width, n_layers, arith;
+  float eps;
+  int64_t side_ld;                                 /* row stride of the token table */
+  const mn_pn_layer* layers;                       /* HOST array [n_layers] */
+  const uint16_t* final_w;
+} mn_pn_model;
+typedef struct mn_pn_state {                       /* HOST arrays [n_layers] of device pointers, fp32 */
+  float* const* k;                                 /* attention: [n_seq, t_max, kv_heads dim]; latent: [n_seq, t_max, ld_latent] */
+  float* const* v;                                 /* attention: [n_seq, t_max, kv_heads vdim] */
+  float* const* conv;                              /* delta: [n_seq, conv - 1, channels] */
+  float* const* lin;                               /* delta: [n_seq, heads, dim, vdim] */
+  int32_t n_seq, t_max;
+} mn_pn_state;
+MN_API size_t mn_sizeof_pn_layer(void);
+MN_API size_t mn_sizeof_pn_model(void);
+MN_API size_t mn_sizeof_pn_state(void);
+/* Row stride of a latent arena: rank + rot rounded up to a multiple of 4 */
+MN_API int mn_pn_latent_ld(int rank, int rot);
+/* One pass of the stack over M rows; rows, row arrays, blk_tab / n_blk, max_len, flags, out and trace as mn_pmix_step (trace: fp32
+ * [n_layers, M, width]); row_tok int32 [M]: the rows' token ids (read by layers with a token input). */
+MN_API size_t mn_pn_workspace_bytes(const mn_pn_model* m, int M);
+MN_API int mn_pn_step(const mn_pn_model* m, const mn_pn_state* st, const float* x, int64_t ldx, int M, const int32_t* row_tok,
+                      const int32_t* row_seq, const int32_t* row_slot, const int32_t* row_back, const int32_t* blk_tab, int n_blk, int max_len,
+                      int flags, float* out, float* trace, void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

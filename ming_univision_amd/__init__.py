@@ -41,6 +41,9 @@ def __getattr__(name):  # lazy: keep `import ming_univision_amd` cheap and torch
     if name in ("ZuzenexDecoder", "ZuzenexForCausalLM"):
         from . import zuzenex
         return getattr(zuzenex, name)
+    if name in ("DaberaxDecoder", "DaberaxForCausalLM"):
+        from . import daberax
+        return getattr(daberax, name)
     if name == "load_model":
         from .infer import load_model
         return load_model

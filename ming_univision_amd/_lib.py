@@ -159,12 +159,31 @@ class HybState(C.Structure):
     _fields_ = [(k, PP) for k in ("k", "v", "lin")] + [("n_seq", C.c_int32), ("t_max", C.c_int32)]
 
 
+class PnLayer(C.Structure):
+    _fields_ = [(k, C.c_int32) for k in ("kind", "heads", "kv_heads", "dim", "vdim", "rot", "kv_rank", "rot_dims", "rot_interleaved", "window",
+                                         "conv", "ff", "side", "has_gate")] + \
+               [(k, C.c_float) for k in ("scale", "softcap", "unit_eps")] + \
+               [(k, C.c_void_p) for k in ("rot_freq", "a_log", "dt_bias", "norm1", "norm2", "side_norm", "w_in", "b_in", "q_norm", "k_norm",
+                                          "w_conv", "mix_norm", "w_ukT", "w_uv", "w_o", "b_o", "w_gate_up", "w_down", "w_side_gate",
+                                          "w_side_proj", "side_table")]
+
+
+class PnModel(C.Structure):
+    _fields_ = [("width", C.c_int32), ("n_layers", C.c_int32), ("arith", C.c_int32), ("eps", C.c_float), ("side_ld", C.c_int64),
+                ("layers", C.POINTER(PnLayer)), ("final_w", C.c_void_p)]
+
+
+class PnState(C.Structure):
+    _fields_ = [(k, PP) for k in ("k", "v", "conv", "lin")] + [("n_seq", C.c_int32), ("t_max", C.c_int32)]
+
+
 # (struct id of mn_struct_layout, its mn_sizeof_* export, the ctypes mirror): checked against the library at load time (`lib()`)
 STRUCTS = ((0, "mn_sizeof_skinny_args", SkinnyArgs), (1, "mn_sizeof_rf_head", RfHead), (2, "mn_sizeof_llm", Llm),
            (3, "mn_sizeof_semdec", SemDec), (4, "mn_sizeof_tp_comm", TpComm), (5, "mn_sizeof_llm_tp", LlmTp),
            (6, "mn_sizeof_seq_layer", SeqLayer), (7, "mn_sizeof_seq_model", SeqModel), (8, "mn_sizeof_seq_state", SeqState),
            (9, "mn_sizeof_pmix_layer", PmixLayer), (10, "mn_sizeof_pmix_model", PmixModel), (11, "mn_sizeof_pmix_state", PmixState),
-           (12, "mn_sizeof_hyb_layer", HybLayer), (13, "mn_sizeof_hyb_model", HybModel), (14, "mn_sizeof_hyb_state", HybState))
+           (12, "mn_sizeof_hyb_layer", HybLayer), (13, "mn_sizeof_hyb_model", HybModel), (14, "mn_sizeof_hyb_state", HybState),
+           (15, "mn_sizeof_pn_layer", PnLayer), (16, "mn_sizeof_pn_model", PnModel), (17, "mn_sizeof_pn_state", PnState))
 
 
 def check_struct_layouts(handle):
@@ -370,6 +389,22 @@ SYMBOLS = {
     "mn_moe_combine_pass_residual": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _i, _i, _p, _i64, _p, _i64, _i, _i, _p]),
     "mn_hyb_workspace_bytes": (_sz, [C.POINTER(HybModel), _i]),
     "mn_hyb_step": (_i, [C.POINTER(HybModel), C.POINTER(HybState), _p, _i64, _i, _p, _p, _p, _p, _i, _p, _i, _i, _i, _p, _p, _p, _sz, _p]),
+    # section 12: post-norm mixed-mixer sequence models
+    "mn_window_pool_attn_blocks_cap": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _f, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f,
+                                            _p, _i64, _p, _i64, _i, _p, _sz, _i, _p]),
+    "mn_sizeof_pn_layer": (_sz, []), "mn_sizeof_pn_model": (_sz, []), "mn_sizeof_pn_state": (_sz, []),
+    "mn_pn_latent_ld": (_i, [_i, _i]),
+    "mn_rotary_frequencies_scaled_host": (_i, [_i, C.c_double, C.c_double, C.c_double, C.c_double, C.c_double, _p]),
+    "mn_rms_scale_add_rows": (_i, [_p, _i64, _p, _i64, _p, _f, _p, _i64, _i, _i, _p]),
+    "mn_gelu_mul_rows": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _i64, _p, _i64, _i, _i, _p]),
+    "mn_proj_norm_rope_append": (_i, [_p, _i64, _i, _i, _i, _i, _i, _p, _p, _f, _i, _i, _p, _f, _p, _p, _p, _i64, _p, _i64, _p, _i64, _i, _p]),
+    "mn_latent_rope_append": (_i, [_p, _i64, _i, _i, _i, _i, _i, _p, _f, _i, _i, _p, _f, _p, _p, _p, _i64, _p, _i64, _i, _p]),
+    "mn_head_sigmoid_gate_rows": (_i, [_p, _i64, _p, _i64, _p, _i64, _i, _i, _i, _p]),
+    "mn_delta_prep_rows": (_i, [_p, _i64, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p, _f, _f, _p, _p, _p, _p, _i64, _p, _i64, _p]),
+    "mn_gated_delta_rows": (_i, [_p, _i64, _p, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _p, _i, _p, _i64, _p]),
+    "mn_head_rms_silu_gate_rows": (_i, [_p, _i64, _p, _f, _p, _i64, _p, _i64, _p, _i64, _i, _i, _i, _p]),
+    "mn_pn_workspace_bytes": (_sz, [C.POINTER(PnModel), _i]),
+    "mn_pn_step": (_i, [C.POINTER(PnModel), C.POINTER(PnState), _p, _i64, _i, _p, _p, _p, _p, _p, _i, _i, _i, _p, _p, _p, _sz, _p]),
     "mn_semdec_step": (_i, [C.POINTER(SemDec), _p, _i, _p, _p, _p, _p, _i, _i64, _p, _p, _p, _sz, _p]),
 }
 
@@ -390,7 +425,7 @@ def lib():
         fn = getattr(handle, name)  # AttributeError if the symbol is missing
         fn.restype = res
         fn.argtypes = args
-    if handle.mn_version() < 128:
+    if handle.mn_version() < 129:
         raise RuntimeError("libmingnative.so is too old")
     check_struct_layouts(handle)
     _lib = handle

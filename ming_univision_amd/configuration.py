@@ -7,6 +7,8 @@
 
   SakinexConfig        <- a decoder-only language model of parallel-mixer layers (windowed attention beside a minGRU, mixture-of-
                           experts feed-forward; no reference counterpart)
+  DaberaxConfig        <- a decoder-only language model of post-norm layers (attention, latent attention or the gated delta rule per
+                          layer, a per-layer token input; no reference counterpart)
   PizitarConfig        <- a decoder-only language model of latent-attention layers (no reference counterpart): config.json keys
                           `architecture`, `width`, `vocab`, `layers`, `canon.taps`, `norm.eps`, `logit_softcap`
 
@@ -596,6 +598,109 @@ def zuzenex_param_shapes(cfg: ZuzenexConfig):
     return s
 
 
+# ---- Daberax ---------------------------------------------------------------------------------------------------------------
+DABERAX_MIXERS = ("attention", "latent_attention", "delta")
+
+
+class DaberaxConfig(_Config):
+    """A stack of layers whose sublayers read the residual stream as it is and whose RESULTS are RMS-normed before they are added.
+    `layers` is a list of dicts(type, mixer, mlp):
+    type  "attention":        mixer dict(heads, kv_heads, dim, vdim, scale, optional rot dict(base, dims, optional scaling dict(factor,
+                              low, high, original)), optional softcap, optional mask dict(size)): biases, RMS norm over the whole q and k
+                              projections, interleaved rotary pairs, soft-capped scores, sliding window, a sigmoid gate per head
+          "latent_attention": mixer dict(heads, dim, rot_dim, vdim, kv_rank, scale, rot dict(base, dims), optional softcap, optional
+                              mask): one normed latent and one rotated key part per token, keys and values are linear maps of the latent
+          "delta":            mixer dict(heads, kv_heads, dim, vdim, conv): the gated delta rule on filtered, unit-length q and k
+    mlp   None or dict(kind="dense", ff)
+    token_side dict(dim): every layer adds a normed projection of gelu(G x) * (its slice of a second embedding row of the token).
+    Every size is read from here or from the tensors; nothing is assumed equal between layers."""
+    model_type = "daberax"
+
+    def __init__(self, width=256, vocab=1024, layers=(), norm=None, token_side=None, logit_scale=1.0, architecture="Daberax", **kwargs):
+        self.architecture = architecture
+        self.width, self.vocab = int(width), int(vocab)
+        self.layers = [copy.deepcopy(dict(ly)) for ly in layers]
+        self.norm = dict(norm or {"eps": 1e-6})
+        self.token_side = dict(token_side) if token_side else None
+        self.logit_scale = float(logit_scale)
+        super().__init__(**kwargs)
+        self.validate()
+
+    eps = property(lambda self: float(self.norm["eps"]))
+    side_dim = property(lambda self: int(self.token_side["dim"]) if self.token_side else 0)
+
+    def validate(self):
+        if self.token_side and int(self.token_side["dim"]) < 1:
+            raise ValueError("token_side.dim must be >= 1")
+        for i, ly in enumerate(self.layers):
+            t = ly.get("type")
+            if t not in DABERAX_MIXERS:
+                raise ValueError(f"layer {i}: unknown mixer type {t!r} (known: {DABERAX_MIXERS})")
+            m = ly["mixer"]
+            need = {"attention": ("heads", "kv_heads", "dim", "vdim", "scale"),
+                    "latent_attention": ("heads", "dim", "rot_dim", "vdim", "kv_rank", "scale"),
+                    "delta": ("heads", "kv_heads", "dim", "vdim", "conv")}[t]
+            for k in need:
+                if k not in m:
+                    raise ValueError(f"layer {i}: mixer lacks {k!r}")
+            if t != "latent_attention" and int(m["heads"]) % int(m["kv_heads"]):
+                raise ValueError(f"layer {i}: {m['heads']} heads do not divide over {m['kv_heads']} key heads")
+            if t == "delta" and int(m["conv"]) < 1:
+                raise ValueError(f"layer {i}: conv must be >= 1")
+            rot = m.get("rot")
+            if t == "latent_attention" and not rot and int(m["rot_dim"]) > 0:
+                raise ValueError(f"layer {i}: latent attention with a rotated part needs rot")
+            if rot and t != "delta":
+                span = int(m["rot_dim"]) if t == "latent_attention" else int(m["dim"])
+                if int(rot["dims"]) % 2 or not (0 <= int(rot["dims"]) <= span):
+                    raise ValueError(f"layer {i}: rot.dims = {rot['dims']} must be even and at most {span}")
+                sc = rot.get("scaling")
+                if sc and not (0 < float(sc["low"]) < float(sc["high"]) and float(sc["factor"]) > 0 and float(sc["original"]) > 0):
+                    raise ValueError(f"layer {i}: rot.scaling {sc}: 0 < low < high, factor > 0, original > 0")
+            if m.get("mask") and int(m["mask"]["size"]) < 1:
+                raise ValueError(f"layer {i}: mask.size must be >= 1")
+            mlp = ly.get("mlp")
+            if mlp is not None and (mlp.get("kind") != "dense" or int(mlp["ff"]) < 1):
+                raise ValueError(f"layer {i}: feed-forward {mlp}: kind 'dense' with ff >= 1")
+
+
+def daberax_param_shapes(cfg: DaberaxConfig):
+    """{tensor name: shape} of a Daberax checkpoint (`l<i>.` per layer, `mix.` the mixer's, `mlp.` the feed-forward's and `side.` the
+    token input's tensors)."""
+    W, V, sd = cfg.width, cfg.vocab, cfg.side_dim
+    s = {"embed": (V, W)}
+    if sd:
+        s["side.embed"] = (V, sd * len(cfg.layers))
+    for i, ly in enumerate(cfg.layers):
+        p, m, mlp, t = f"l{i}.", ly["mixer"], ly.get("mlp"), ly["type"]
+        H, d, e = int(m["heads"]), int(m["dim"]), int(m["vdim"])
+        s[p + "norm1"] = (W,)
+        if t == "attention":
+            G = int(m["kv_heads"])
+            s[p + "mix.q"], s[p + "mix.k"], s[p + "mix.v"] = (H * d, W), (G * d, W), (G * e, W)
+            s[p + "mix.q.b"], s[p + "mix.k.b"], s[p + "mix.v.b"], s[p + "mix.o.b"] = (H * d,), (G * d,), (G * e,), (W,)
+            s[p + "mix.q.norm"], s[p + "mix.k.norm"], s[p + "mix.g"] = (H * d,), (G * d,), (H, W)
+        elif t == "latent_attention":
+            r, R = int(m["rot_dim"]), int(m["kv_rank"])
+            s[p + "mix.q"], s[p + "mix.dkv"], s[p + "mix.dkv.norm"] = (H * (d + r), W), (R + r, W), (R,)
+            s[p + "mix.uk"], s[p + "mix.uv"] = (H * d, R), (H * e, R)
+        else:
+            G, taps = int(m["kv_heads"]), int(m["conv"])
+            for n, rows in (("q", G * d), ("k", G * d), ("v", H * e)):
+                s[p + "mix." + n], s[p + "mix." + n + ".conv"] = (rows, W), (rows, taps)
+            s[p + "mix.b"], s[p + "mix.a"], s[p + "mix.A_log"], s[p + "mix.dt_bias"] = (H, W), (H, W), (H,), (H,)
+            s[p + "mix.norm"], s[p + "mix.g"] = (e,), (H * e, W)
+        s[p + "mix.o"] = (W, H * e)
+        if mlp is not None:
+            ff = int(mlp["ff"])
+            s[p + "norm2"] = (W,)
+            s[p + "mlp.gate"], s[p + "mlp.up"], s[p + "mlp.down"] = (ff, W), (ff, W), (W, ff)
+        if sd:
+            s[p + "side.gate"], s[p + "side.proj"], s[p + "side.norm"] = (sd, W), (W, sd), (W,)
+    s["final.norm"], s["head"] = (W,), (V, W)
+    return s
+
+
 # ---- registry: which configuration class a config.json belongs to -------------------------------------------------------------
 def _is_pizitar(d):
     return d.get("architecture") == "Pizitar" or d.get("model_type") == "pizitar"
@@ -609,11 +714,16 @@ def _is_zuzenex(d):
     return d.get("architecture") == "Zuzenex" or d.get("model_type") == "zuzenex"
 
 
+def _is_daberax(d):
+    return d.get("architecture") == "Daberax" or d.get("model_type") == "daberax"
+
+
 def _is_ming_univision(d):
     return "llm_config" in d or d.get("model_type") in ("bailingmm", "ming_univision")
 
 
 MODEL_REGISTRY = [("pizitar", _is_pizitar, PizitarConfig), ("sakinex", _is_sakinex, SakinexConfig), ("zuzenex", _is_zuzenex, ZuzenexConfig),
+                  ("daberax", _is_daberax, DaberaxConfig),
                   ("ming_univision", _is_ming_univision, MingUniVisionConfig)]
 
 

@@ -162,16 +162,34 @@ extern "C" int mn_struct_layout(int which, size_t* offsets, int cap) {
       F(k) F(v) F(lin) F(n_seq) F(t_max)
 #undef F
   };
+  static const size_t pn_layer[] = {
+#define F(f) MN_OFF(mn_pn_layer, f)
+      F(kind) F(heads) F(kv_heads) F(dim) F(vdim) F(rot) F(kv_rank) F(rot_dims) F(rot_interleaved) F(window) F(conv) F(ff) F(side) F(has_gate)
+      F(scale) F(softcap) F(unit_eps) F(rot_freq) F(a_log) F(dt_bias) F(norm1) F(norm2) F(side_norm) F(w_in) F(b_in) F(q_norm) F(k_norm)
+      F(w_conv) F(mix_norm) F(w_ukT) F(w_uv) F(w_o) F(b_o) F(w_gate_up) F(w_down) F(w_side_gate) F(w_side_proj) F(side_table)
+#undef F
+  };
+  static const size_t pn_model[] = {
+#define F(f) MN_OFF(mn_pn_model, f)
+      F(width) F(n_layers) F(arith) F(eps) F(side_ld) F(layers) F(final_w)
+#undef F
+  };
+  static const size_t pn_state[] = {
+#define F(f) MN_OFF(mn_pn_state, f)
+      F(k) F(v) F(conv) F(lin) F(n_seq) F(t_max)
+#undef F
+  };
   const size_t* tab[] = {skinny, rf, llm, semdec, comm, llm_tp, seq_layer, seq_model, seq_state, pmix_layer, pmix_model, pmix_state,
-                         hyb_layer, hyb_model, hyb_state};
+                         hyb_layer, hyb_model, hyb_state, pn_layer, pn_model, pn_state};
   const int cnt[] = {(int)(sizeof(skinny) / sizeof(size_t)), (int)(sizeof(rf) / sizeof(size_t)), (int)(sizeof(llm) / sizeof(size_t)),
                      (int)(sizeof(semdec) / sizeof(size_t)), (int)(sizeof(comm) / sizeof(size_t)), (int)(sizeof(llm_tp) / sizeof(size_t)),
                      (int)(sizeof(seq_layer) / sizeof(size_t)), (int)(sizeof(seq_model) / sizeof(size_t)),
                      (int)(sizeof(seq_state) / sizeof(size_t)), (int)(sizeof(pmix_layer) / sizeof(size_t)),
                      (int)(sizeof(pmix_model) / sizeof(size_t)), (int)(sizeof(pmix_state) / sizeof(size_t)),
                      (int)(sizeof(hyb_layer) / sizeof(size_t)), (int)(sizeof(hyb_model) / sizeof(size_t)),
-                     (int)(sizeof(hyb_state) / sizeof(size_t))};
-  MN_CHECK_ARG(which >= 0 && which < 15, "mn_struct_layout: unknown struct id");
+                     (int)(sizeof(hyb_state) / sizeof(size_t)), (int)(sizeof(pn_layer) / sizeof(size_t)),
+                     (int)(sizeof(pn_model) / sizeof(size_t)), (int)(sizeof(pn_state) / sizeof(size_t))};
+  MN_CHECK_ARG(which >= 0 && which < 18, "mn_struct_layout: unknown struct id");
   for (int i = 0; i < cnt[which] && i < cap; ++i) offsets[i] = tab[which][i];
   return cnt[which];
 }

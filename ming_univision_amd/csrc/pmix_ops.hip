@@ -504,7 +504,11 @@ struct AttnTArgs {
   float* out; int64_t ldo; bf16_t* out16; int64_t ldo16;
   float* part;
   const float* sink;    // optional fp32 [H]: exp(sink[h]) joins the softmax's denominator of head h (no key, no value)
+  float cap;            // > 0: every score s becomes cap * tanh(s / cap) before the softmax
+  int64_t ldk, ldv;     // row strides of the key and value arenas (>= G * dim, G * vdim): a value arena may be a view into the key arena
 };
+
+__device__ __forceinline__ float soft_cap(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 
 // 1 / (the softmax's normaliser) of a vector with running maximum m and sum l (of exp(score - m)), the head's sink included:
 // numerator and denominator are both taken relative to max(m, sink)
@@ -548,8 +552,8 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(AttnTArgs a) {
   }
   if (tid < AQ) { st_m[tid] = -INFINITY; st_l[tid] = 0.f; st_a[tid] = 0.f; }
   const int Gd = a.G * a.dim, Gv = a.G * a.vdim;
-  const float* kb = a.k + ((int64_t)seq * a.t_max + tF) * Gd + (int64_t)g * a.dim;
-  const float* vb = a.v + ((int64_t)seq * a.t_max + tF) * Gv + (int64_t)g * a.vdim;
+  const float* kb = a.k + ((int64_t)seq * a.t_max + tF) * a.ldk + (int64_t)g * a.dim;
+  const float* vb = a.v + ((int64_t)seq * a.t_max + tF) * a.ldv + (int64_t)g * a.vdim;
   const float* pkb = a.pk ? a.pk + (int64_t)seq * a.n_pool_max * Gd + (int64_t)g * a.dim : nullptr;
   const float* pvb = a.pv ? a.pv + (int64_t)seq * a.n_pool_max * Gv + (int64_t)g * a.vdim : nullptr;
   constexpr int NCB = 2;                    // column blocks of 256: vdim <= 512
@@ -565,7 +569,7 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(AttnTArgs a) {
     {  // ---- scores ----
       const int key = tid >> 2, part = tid & 3, j = j0 + key;
       const bool valid = key < nt;
-      const float* kp = !valid ? kb : (j < nbL ? pkb + (int64_t)j * Gd : kb + (int64_t)(j - nbL) * Gd);
+      const float* kp = !valid ? kb : (j < nbL ? pkb + (int64_t)j * Gd : kb + (int64_t)(j - nbL) * a.ldk);
       float s[AQ];
 #pragma unroll
       for (int i = 0; i < AQ; ++i) s[i] = 0.f;
@@ -607,7 +611,7 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(AttnTArgs a) {
         if ((i & 3) == part) {
           const int pos = pos0 + i / Rc;
           const bool see = valid && i < nqv && (j < nbL ? j < win_nb(pos, a.window, a.pool) : (t >= win_t0(pos, a.window) && t <= pos));
-          sc[i * AKT + key] = see ? v : -INFINITY;
+          sc[i * AKT + key] = see ? soft_cap(v, a.cap) : -INFINITY;
         }
       }
     }
@@ -642,7 +646,7 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(AttnTArgs a) {
 #pragma unroll
           for (int u = 0; u < PRE; ++u) {
             const int jj = jj0 + u * nsub, j = j0 + jj;
-            vv[u] = jj < nt ? (j < nbL ? pvb + (int64_t)j * Gv : vb + (int64_t)(j - nbL) * Gv)[c0 + c] : 0.f;
+            vv[u] = jj < nt ? (j < nbL ? pvb + (int64_t)j * Gv : vb + (int64_t)(j - nbL) * a.ldv)[c0 + c] : 0.f;
           }
 #pragma unroll
           for (int u = 0; u < PRE; ++u) {
@@ -748,16 +752,16 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(AttnTArgs a) {
 #pragma unroll
   for (int c = 0; c < NBV; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int Gd = a.G * a.dim, Gv = a.G * a.vdim;
-  const float* kb = a.k + ((int64_t)seq * a.t_max + tF) * Gd + (int64_t)g * a.dim;
-  const float* vb = a.v + ((int64_t)seq * a.t_max + tF) * Gv + (int64_t)g * a.vdim;
+  const float* kb = a.k + ((int64_t)seq * a.t_max + tF) * a.ldk + (int64_t)g * a.dim;
+  const float* vb = a.v + ((int64_t)seq * a.t_max + tF) * a.ldv + (int64_t)g * a.vdim;
   const float* pkb = a.pk ? a.pk + (int64_t)seq * a.n_pool_max * Gd + (int64_t)g * a.dim : nullptr;
   const float* pvb = a.pv ? a.pv + (int64_t)seq * a.n_pool_max * Gv + (int64_t)g * a.vdim : nullptr;
   f32x4 vk[NBD], vv[NBV];
   auto fetch = [&](int tile) {
     const int k0 = tile * KT;
-    load16<NBD>(vk, a.dim, tid, [&](int j) { const int jj = min(k0 + j, nk - 1); return jj < nbL ? pkb + (int64_t)jj * Gd : kb + (int64_t)(jj - nbL) * Gd; },
+    load16<NBD>(vk, a.dim, tid, [&](int j) { const int jj = min(k0 + j, nk - 1); return jj < nbL ? pkb + (int64_t)jj * Gd : kb + (int64_t)(jj - nbL) * a.ldk; },
                 [&](int j) { return k0 + j < nk; });
-    load16<NBV>(vv, a.vdim, tid, [&](int j) { const int jj = min(k0 + j, nk - 1); return jj < nbL ? pvb + (int64_t)jj * Gv : vb + (int64_t)(jj - nbL) * Gv; },
+    load16<NBV>(vv, a.vdim, tid, [&](int j) { const int jj = min(k0 + j, nk - 1); return jj < nbL ? pvb + (int64_t)jj * Gv : vb + (int64_t)(jj - nbL) * a.ldv; },
                 [&](int j) { return k0 + j < nk; });
   };
   if (t0 < t1) fetch(t0);
@@ -786,7 +790,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(AttnTArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int o = (4 * g4 + i) * LDS_S + c16;
-      float sc = (Sp[o] + Sp[16 * LDS_S + o]) + (Sp[32 * LDS_S + o] + Sp[48 * LDS_S + o]);
+      float sc = soft_cap((Sp[o] + Sp[16 * LDS_S + o]) + (Sp[32 * LDS_S + o] + Sp[48 * LDS_S + o]), a.cap);
       const bool see = j < nk && (j < nbL ? j < my_nb[i] : (tok >= my_t0[i] && tok <= mypos[i]));
       if (!see) sc = -INFINITY;
       const float mnew = fmaxf(mrun[i], row16_max(sc));
@@ -1229,6 +1233,22 @@ extern "C" int mn_window_pool_attn_blocks_sink(const float* q, int64_t ldq, cons
                                                const int32_t* blk_tab, int n_blk, int one_row, int H, int G, int dim, int vdim, int t_max,
                                                int n_pool_max, int window, int pool, float out_scale, float* out, int64_t ldo, uint16_t* out16,
                                                int64_t ldo16, int nsplit, void* workspace, size_t workspace_bytes, int variant, void* stream) {
+  return mn_window_pool_attn_blocks_cap(q, ldq, k_arena, 0, v_arena, 0, pk, pv, sink, 0.0f, row_seq, row_slot, blk_tab, n_blk, one_row, H, G, dim,
+                                        vdim, t_max, n_pool_max, window, pool, out_scale, out, ldo, out16, ldo16, nsplit, workspace,
+                                        workspace_bytes, variant, stream);
+}
+
+extern "C" int mn_window_pool_attn_blocks_cap(const float* q, int64_t ldq, const float* k_arena, int64_t ldk, const float* v_arena, int64_t ldv,
+                                              const float* pk, const float* pv, const float* sink, float softcap, const int32_t* row_seq,
+                                              const int32_t* row_slot, const int32_t* blk_tab, int n_blk, int one_row, int H, int G, int dim,
+                                              int vdim, int t_max, int n_pool_max, int window, int pool, float out_scale, float* out, int64_t ldo,
+                                              uint16_t* out16, int64_t ldo16, int nsplit, void* workspace, size_t workspace_bytes, int variant,
+                                              void* stream) {
+  if (ldk <= 0) ldk = (int64_t)G * dim;
+  if (ldv <= 0) ldv = (int64_t)G * vdim;
+  MN_CHECK_ARG(ldk >= (int64_t)G * dim && ldv >= (int64_t)G * vdim && ((dim % 4) != 0 || (ldk % 4) == 0) && ((vdim % 4) != 0 || (ldv % 4) == 0) &&
+                   softcap >= 0.0f,
+               "mn_window_pool_attn_blocks: arena row strides below a row, or no multiple of 4 under heads that are; or a negative soft cap");
   if (variant < 0) variant = (!one_row && dim <= 256 && vdim <= 256) ? MN_WINDOW_ATTN_MFMA : MN_WINDOW_ATTN_VALU;
   MN_CHECK_ARG(q && k_arena && v_arena && row_seq && row_slot && (out || out16) && n_blk >= 1 && H >= 1 && G >= 1 && (H % G) == 0 && dim >= 1 &&
                    vdim >= 1 && vdim <= 512 && t_max >= 1 && window >= 0 && pool >= 0 && nsplit >= 1 && nsplit <= 64,
@@ -1240,7 +1260,7 @@ extern "C" int mn_window_pool_attn_blocks_sink(const float* q, int64_t ldq, cons
   MN_CHECK_ARG(nsplit == 1 || (workspace && workspace_bytes >= mn_window_attn_workspace_bytes(n_blk, H, G, vdim, one_row, nsplit)),
                "mn_window_pool_attn_blocks: workspace too small");
   AttnTArgs a{q, ldq, k_arena, v_arena, pool ? pk : nullptr, pool ? pv : nullptr, row_seq, row_slot, one_row ? nullptr : blk_tab, H, G, dim, vdim,
-              t_max, n_pool_max, window, pool, sh.rows, sh.hpc, nsplit, out_scale, out, ldo, out16, ldo16, (float*)workspace, sink};
+              t_max, n_pool_max, window, pool, sh.rows, sh.hpc, nsplit, out_scale, out, ldo, out16, ldo16, (float*)workspace, sink, softcap, ldk, ldv};
   MN_CHECK_ARG(variant == MN_WINDOW_ATTN_VALU || (variant == MN_WINDOW_ATTN_MFMA && !one_row && dim <= 256 && vdim <= 256),
                "mn_window_pool_attn_blocks: the matrix-core kernel takes runs of rows with dim, vdim <= 256");
   if (variant == MN_WINDOW_ATTN_MFMA) {
@@ -1262,7 +1282,7 @@ extern "C" int mn_window_pool_attn_blocks_sink(const float* q, int64_t ldq, cons
   }
   const size_t lds = ((size_t)sh.aq * dim + 2 * (size_t)sh.aq * AKT + 3 * sh.aq + (size_t)sh.aq * 256) * sizeof(float);
   MN_CHECK_ARG(lds <= 64 * 1024, "mn_window_pool_attn_blocks: dim=%d too large", dim);
-  const bool vec = (dim % 4) == 0 && (ldq % 4) == 0 && (((uintptr_t)q | (uintptr_t)k_arena | (uintptr_t)pk) & 15) == 0;
+  const bool vec = (dim % 4) == 0 && (ldq % 4) == 0 && (ldk % 4) == 0 && (((uintptr_t)q | (uintptr_t)k_arena | (uintptr_t)pk) & 15) == 0;
   const dim3 grid((unsigned)n_blk, (unsigned)(G * sh.chunks), (unsigned)nsplit);
   hipStream_t st = mn_stream(stream);
   if (sh.aq == 4) {

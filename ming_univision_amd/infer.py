@@ -43,7 +43,7 @@ def load_safetensors_dir(path):
 
 def load_model(path, dtype="bf16", device="cuda", **kw):
     """The served model of a checkpoint directory, its class chosen by config.json (configuration.MODEL_REGISTRY):
-    "pizitar" -> PizitarForCausalLM, "sakinex" -> SakinexForCausalLM, "zuzenex" -> ZuzenexForCausalLM (dtype "bf16" | "f32" = the matrix-product arithmetic; kw: t_max,
+    "pizitar" -> PizitarForCausalLM, "sakinex" -> SakinexForCausalLM, "zuzenex" -> ZuzenexForCausalLM, "daberax" -> DaberaxForCausalLM (dtype "bf16" | "f32" = the matrix-product arithmetic; kw: t_max,
     eos_token_id),
     "ming_univision" -> MingUniVisionInfer (dtype = the weight format)."""
     from .configuration import config_from_pretrained
@@ -57,6 +57,9 @@ def load_model(path, dtype="bf16", device="cuda", **kw):
     if name == "zuzenex":
         from .zuzenex import ZuzenexForCausalLM
         return ZuzenexForCausalLM.from_pretrained(path, device=device, arith=dtype, **kw)
+    if name == "daberax":
+        from .daberax import DaberaxForCausalLM
+        return DaberaxForCausalLM.from_pretrained(path, device=device, arith=dtype, **kw)
     return MingUniVisionInfer(path, dtype=dtype, device=device, **kw)
 
 

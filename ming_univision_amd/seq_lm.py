@@ -4,7 +4,8 @@ passes, the vocabulary projection and the picks, a decode step captured as a HIP
 A decoder class (`pizitar.PizitarDecoder`, `sakinex.SakinexDecoder`, `zuzenex.ZuzenexDecoder`) owns its weights, caches and states and gives
     step(x, row_seq, row_slot, row_back, row_len, blk_tab, max_len, out, trace, ws, distinct)   one pass over <= max_rows() rows
     _workspace_bytes(rows, max_len), ensure_sequences(n), release_sequences(n), n_trace (residual streams a trace holds)
-(a decoder with a `chunk_rows` attribute also gets chunk_tab = its rows cut into chunks of that many rows of one sequence)
+(a decoder with a `chunk_rows` attribute also gets chunk_tab = its rows cut into chunks of that many rows of one sequence; a decoder
+whose layers read the token ids themselves sets `needs_tokens` and gets row_tok = the rows' ids as an int32 device array)
 and inherits the rest from `SeqDecoder`; its generation entry point derives from `SeqCausalLM`.
 """
 import ctypes as C
@@ -34,12 +35,18 @@ class SeqDecoder:
             self._ws[key] = torch.empty(need, dtype=torch.uint8, device=self.device)
         return self._ws[key]
 
-    def forward_spans(self, x, spans, trace=False):
+    needs_tokens = False
+
+    def forward_spans(self, x, spans, trace=False, tokens=None):
         """Rows of several sequences through the stack: spans = [(cache sequence, rows, tokens it already holds)] in row order,
-        x fp32 [sum rows, width].  Runs in passes of <= max_rows() rows; a sequence cut by a pass boundary continues in the next
-        pass.  Returns the final-norm hidden states [rows, width] (and the per-layer residual streams when trace)."""
+        x fp32 [sum rows, width]; tokens: the rows' ids (a decoder with `needs_tokens` reads them).  Runs in passes of <= max_rows()
+        rows; a sequence cut by a pass boundary continues in the next pass.  Returns the final-norm hidden states [rows, width] (and
+        the per-layer residual streams when trace)."""
         M = x.shape[0]
         assert sum(n for _, n, _ in spans) == M
+        if self.needs_tokens:
+            assert tokens is not None and tokens.numel() == M, "this decoder's layers read the token ids: pass tokens="
+            tokens = tokens.reshape(-1).to(self.device, torch.int32).contiguous()
         out = torch.empty(M, self.cfg.width, dtype=torch.float32, device=self.device)
         tr = torch.empty(self.n_trace, M, self.cfg.width, dtype=torch.float32, device=self.device) if trace else None
         starts = np.cumsum([0] + [n for _, n, _ in spans])
@@ -54,14 +61,15 @@ class SeqDecoder:
                 ptr_tr = torch.empty(self.n_trace, r1 - r0, self.cfg.width, dtype=torch.float32, device=self.device)
             self.step(x[r0:r1], dev["row_seq"], dev["row_slot"], dev["row_back"], dev["row_len"], dev["blk_tab"], tabs["max_len"],
                       out=out[r0:r1], trace=ptr_tr, distinct=all(n == 1 for _, n, _ in part),
-                      **({"chunk_tab": dev["chunk_tab"]} if "chunk_tab" in dev else {}))
+                      **({"chunk_tab": dev["chunk_tab"]} if "chunk_tab" in dev else {}),
+                      **({"row_tok": tokens[r0:r1]} if self.needs_tokens else {}))
             if trace:
                 tr[:, r0:r1] = ptr_tr
         return (out, tr) if trace else out
 
     def prefill(self, ids, seq=0, past=0):
         """Tokens ids (int tensor [T]) of ONE sequence from slot `past`; returns the hidden states [T, width]."""
-        return self.forward_spans(self.embed(ids), [(seq, int(ids.numel()), past)])
+        return self.forward_spans(self.embed(ids), [(seq, int(ids.numel()), past)], tokens=ids)
 
     def decode_tables(self, B):
         """Static per-row tables of a lock-step decode step of B sequences (one row each): (row_back, blk_tab)."""
@@ -118,17 +126,21 @@ class DecodeGraph:
         self.back, self.blk = dec.decode_tables(B)
         self.x = torch.zeros(B, dec.cfg.width, dtype=torch.float32, device=dec.device)
         self.out = torch.empty(B, dec.cfg.width, dtype=torch.float32, device=dec.device)
+        self.tok = torch.zeros(B, dtype=torch.int32, device=dec.device) if dec.needs_tokens else None
         n = int(dec._workspace_bytes(B, dec.t_max))
         self.ws = torch.empty(n, dtype=torch.uint8, device=dec.device)
         self.bound, self.graph = 0, None
 
     def _body(self):
-        self.dec.step(self.x, self.row_seq, self.slot, self.back, self.len, self.blk, self.bound, out=self.out, ws=self.ws, distinct=True)
+        self.dec.step(self.x, self.row_seq, self.slot, self.back, self.len, self.blk, self.bound, out=self.out, ws=self.ws, distinct=True,
+                      **({"row_tok": self.tok} if self.tok is not None else {}))
         check(lib().mn_rows_advance(ptr(self.slot), ptr(self.len), None, self.B, 1, current_stream()), "mn_rows_advance")
 
-    def run(self, x, max_len):
-        """x fp32 [B, width]: the new tokens' embeddings; max_len: host upper bound of the lengths after this step.
-        Returns the hidden states [B, width] (a fixed buffer, overwritten by the next run)."""
+    def run(self, x, max_len, tokens=None):
+        """x fp32 [B, width]: the new tokens' embeddings (tokens: their ids, for a decoder with `needs_tokens`); max_len: host upper
+        bound of the lengths after this step.  Returns the hidden states [B, width] (a fixed buffer, overwritten by the next run)."""
+        if self.tok is not None:
+            self.tok.copy_(tokens.reshape(-1))
         if self.graph is None or max_len > self.bound:
             self.bound = min(self.dec.t_max, (max_len + self.span - 1) // self.span * self.span)
             self.graph = torch.cuda.CUDAGraph()
@@ -168,7 +180,7 @@ class SeqCausalLM:
         seqs = [self.slots.alloc() for _ in range(B)]
         try:
             ids = torch.tensor([t for p in prompts for t in p], dtype=torch.long, device=dev)
-            hid = dec.forward_spans(dec.embed(ids), [(s, n, 0) for s, n in zip(seqs, lens)])
+            hid = dec.forward_spans(dec.embed(ids), [(s, n, 0) for s, n in zip(seqs, lens)], tokens=ids)
             last = torch.tensor(np.cumsum(lens) - 1, dtype=torch.long, device=dev)
             hidden = hid[last].contiguous()
             row_seq = torch.tensor(seqs, dtype=torch.int32, device=dev)
@@ -189,9 +201,10 @@ class SeqCausalLM:
                 if i + 1 == max_new_tokens:
                     break
                 if graph is not None:
-                    hidden = graph.run(dec.embed(tok), max(lens) + i + 1)
+                    hidden = graph.run(dec.embed(tok), max(lens) + i + 1, tokens=tok)
                 else:
-                    hidden = dec.step(dec.embed(tok), row_seq, slot, back, ln, blk, max(lens) + i + 1, distinct=True)
+                    hidden = dec.step(dec.embed(tok), row_seq, slot, back, ln, blk, max(lens) + i + 1, distinct=True,
+                                      **({"row_tok": tok.to(torch.int32)} if dec.needs_tokens else {}))
                     check(lib().mn_rows_advance(ptr(slot), ptr(ln), None, B, 1, current_stream()), "mn_rows_advance")
             out = torch.stack(toks, 1).tolist()
         finally:

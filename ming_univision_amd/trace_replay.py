@@ -8,7 +8,7 @@ among these tokens whose logits are written, for all entries in order, to OUT/<n
 Requests named in `end` give their cache sequence back after the step.  `done <n>` is printed after every step.
 
 The model class comes from config.json through the framework's registry (`infer.load_model`); the step runs the served path:
-`decoder.forward_spans` (mn_seq_step, mn_pmix_step or mn_hyb_step), the decoder's arenas and states and `sequences.SequenceSlots`.  Nothing is sampled.
+`decoder.forward_spans` (mn_seq_step, mn_pmix_step, mn_hyb_step or mn_pn_step), the decoder's arenas and states and `sequences.SequenceSlots`.  Nothing is sampled.
 --dtype bfloat16 is the serving arithmetic (bf16 MFMA products above 8 rows, fp32 elsewhere), float32 is fp32 FMA everywhere.
 """
 import argparse
@@ -47,7 +47,7 @@ def replay(model, out_dir, lines, emit):
             r0 += n
         if spans:
             ids = torch.tensor(toks, dtype=torch.long, device=dec.device)
-            hidden = dec.forward_spans(dec.embed(ids), spans)
+            hidden = dec.forward_spans(dec.embed(ids), spans, tokens=ids)
             if want:
                 rows = hidden[torch.tensor(want, dtype=torch.long, device=dec.device)]
                 logits = dec.logits(rows).cpu().numpy().astype("<f4")
