@@ -213,3 +213,96 @@ def forward(cfg, sd, tokens):
         streams.append(x)
     y = rms(x, eps) * f64(sd["final.norm"])
     return (y @ f64(sd["head"]).T) * float(cfg.get("logit_scale", 1.0)), torch.stack(streams)
+
+
+# ---- small models for the tests ----------------------------------------------------------------------------------------------------
+def dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def attention_layer(heads=4, kv_heads=2, dim=16, vdim=16, scale=0.25, rot=(10000.0, 16), scaling=None, softcap=None, window=None, mlp=None):
+    m = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale)
+    if rot:
+        m["rot"] = {"base": rot[0], "dims": rot[1]}
+        if scaling:
+            m["rot"]["scaling"] = dict(zip(("factor", "low", "high", "original"), scaling))
+    if softcap:
+        m["softcap"] = softcap
+    if window:
+        m["mask"] = {"size": window}
+    return {"type": "attention", "mixer": m, "mlp": mlp}
+
+
+def latent_layer(heads=4, dim=8, rot_dim=8, vdim=12, kv_rank=24, scale=0.25, base=10000.0, softcap=None, window=None, mlp=None):
+    m = dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=kv_rank, scale=scale, rot={"base": base, "dims": rot_dim})
+    if softcap:
+        m["softcap"] = softcap
+    if window:
+        m["mask"] = {"size": window}
+    return {"type": "latent_attention", "mixer": m, "mlp": mlp}
+
+
+def delta_layer(heads=4, kv_heads=2, dim=16, vdim=16, conv=4, mlp=None):
+    return {"type": "delta", "mixer": dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, conv=conv), "mlp": mlp}
+
+
+def small_config(layers, width=64, vocab=80, side=6, logit_scale=0.5, eps=1e-5):
+    cfg = {"architecture": "Daberax", "width": width, "vocab": vocab, "norm": {"eps": eps}, "layers": layers, "logit_scale": logit_scale}
+    if side:
+        cfg["token_side"] = {"dim": side}
+    return cfg
+
+
+def param_shapes(cfg):
+    W, V = cfg["width"], cfg["vocab"]
+    side = (cfg.get("token_side") or {}).get("dim", 0)
+    s = {"embed": (V, W), "final.norm": (W,), "head": (V, W)}
+    if side:
+        s["side.embed"] = (V, side * len(cfg["layers"]))
+    for i, ly in enumerate(cfg["layers"]):
+        p, m, t = f"l{i}.", ly["mixer"], ly["type"]
+        H, d, e = m["heads"], m["dim"], m["vdim"]
+        s.update({p + "norm1": (W,), p + "mix.o": (W, H * e)})
+        if t == "attention":
+            G = m["kv_heads"]
+            s.update({p + "mix.q": (H * d, W), p + "mix.k": (G * d, W), p + "mix.v": (G * e, W), p + "mix.q.b": (H * d,), p + "mix.k.b": (G * d,),
+                      p + "mix.v.b": (G * e,), p + "mix.o.b": (W,), p + "mix.q.norm": (H * d,), p + "mix.k.norm": (G * d,), p + "mix.g": (H, W)})
+        elif t == "latent_attention":
+            r, R = m["rot_dim"], m["kv_rank"]
+            s.update({p + "mix.q": (H * (d + r), W), p + "mix.dkv": (R + r, W), p + "mix.dkv.norm": (R,), p + "mix.uk": (H * d, R),
+                      p + "mix.uv": (H * e, R)})
+        else:
+            G, taps = m["kv_heads"], m["conv"]
+            s.update({p + "mix.q": (G * d, W), p + "mix.k": (G * d, W), p + "mix.v": (H * e, W), p + "mix.q.conv": (G * d, taps),
+                      p + "mix.k.conv": (G * d, taps), p + "mix.v.conv": (H * e, taps), p + "mix.b": (H, W), p + "mix.a": (H, W),
+                      p + "mix.A_log": (H,), p + "mix.dt_bias": (H,), p + "mix.norm": (e,), p + "mix.g": (H * e, W)})
+        if ly.get("mlp") is not None:
+            ff = ly["mlp"]["ff"]
+            s.update({p + "norm2": (W,), p + "mlp.gate": (ff, W), p + "mlp.up": (ff, W), p + "mlp.down": (W, ff)})
+        if side:
+            s.update({p + "side.gate": (side, W), p + "side.proj": (W, side), p + "side.norm": (W,)})
+    return s
+
+
+def random_weights(cfg, seed=0):
+    """bf16 tensors under the checkpoint's names: norm weights around 1, decays spread between slow and fast, biases that matter."""
+    g = torch.Generator().manual_seed(seed)
+    sd = {}
+    for k, shp in param_shapes(cfg).items():
+        r = torch.randn(shp, generator=g)
+        if k in ("embed", "side.embed"):
+            t = r
+        elif "norm" in k:
+            t = 1.0 + 0.1 * r
+        elif k.endswith("A_log"):
+            t = -1.0 + r
+        elif k.endswith("dt_bias"):
+            t = r
+        elif k.endswith(".conv"):
+            t = 0.6 * r
+        elif len(shp) == 1:
+            t = 0.3 * r
+        else:
+            t = 1.3 * r * shp[-1] ** -0.5
+        sd[k] = t.to(torch.bfloat16)
+    return sd
