@@ -30,7 +30,7 @@ def test_config_and_registry(tmp_path):
     (tmp_path / "config.json").write_text(json.dumps({"architecture": "Other"}))
     with pytest.raises(ValueError):
         config_from_pretrained(str(tmp_path))
-    assert [n for n, _, _ in MODEL_REGISTRY] == ["pizitar", "sakinex", "zuzenex", "ming_univision"]
+    assert [n for n, _, _ in MODEL_REGISTRY] == ["pizitar", "sakinex", "zuzenex", "daberax", "ming_univision"]
 
 
 @pytest.mark.parametrize("edit", [
