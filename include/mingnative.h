@@ -933,6 +933,9 @@ MN_API int mn_window_pool_attn(const float* q, int64_t ldq, const float* k_arena
  * mn_window_attn_workspace_bytes).  vdim <= 512. */
 MN_API int mn_window_attn_block_rows(void);
 MN_API int mn_window_attn_splits(int n_blk, int H, int G, int one_row, int max_keys);
+/* the same for a kernel whose key tiles hold key_tile keys (64: the fp32 FMA kernel, what mn_window_attn_splits assumes; 16: the
+ * matrix-core kernel, which decode rows take when their values lie inside their keys) */
+MN_API int mn_window_attn_splits_tile(int n_blk, int H, int G, int one_row, int max_keys, int key_tile);
 MN_API size_t mn_window_attn_workspace_bytes(int n_blk, int H, int G, int vdim, int one_row, int nsplit);
 MN_API int mn_window_pool_attn_blocks(const float* q, int64_t ldq, const float* k_arena, const float* v_arena, const float* pk,
                                       const float* pv, const int32_t* row_seq, const int32_t* row_slot, const int32_t* blk_tab, int n_blk,

@@ -366,6 +366,7 @@ SYMBOLS = {
     "mn_pmix_step": (_i, [C.POINTER(PmixModel), C.POINTER(PmixState), _p, _i64, _i, _p, _p, _p, _p, _i, _i, _i, _p, _p, _p, _sz, _p]),
     "mn_window_attn_block_rows": (_i, []),
     "mn_window_attn_splits": (_i, [_i, _i, _i, _i, _i]),
+    "mn_window_attn_splits_tile": (_i, [_i, _i, _i, _i, _i, _i]),
     "mn_window_attn_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
     "mn_window_pool_attn_blocks": (_i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _p, _i64, _p, _i64, _i,
                                         _p, _sz, _p]),

@@ -704,16 +704,19 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(AttnTArgs a) {
 //            visibility and keep the same running maximum / sum
 //   values   O[16 q, vdim] += P V: the weights go through LDS into the A-operand layout, wave w owns the 16-column blocks w, w + 4, ..
 // NBD / NBV: 64-value blocks of a key / a value (zero padded).  Key splits write the same partial layout as the tiled form.
-template <int NBD, int NBV>
+// VK: the values are the first columns of the keys (one key/value head whose value arena is a view of the key arena — latent
+// attention): the staged key tile serves both products and no value tile is loaded; NBV <= NBD.  Without a table of runs (decode
+// rows) workgroup b takes row b and its up to 16 query heads.
+template <int NBD, int NBV, bool VK = false>
 __global__ __launch_bounds__(256) void window_attn_mfma_kernel(AttnTArgs a) {
-  constexpr int KT = 16, LDP = 20, LDS_S = 17, DP = 64 * NBD, VP = 64 * NBV, LDK = DP + 4, LDV = VP + 4, DQ = DP / 4, AQ = 16;
+  constexpr int KT = 16, LDP = 20, LDS_S = 17, DP = 64 * NBD, VP = 64 * NBV, LDK = DP + 4, LDV = VK ? LDK : VP + 4, DQ = DP / 4, AQ = 16;
   extern __shared__ float lds[];
   const int tid = threadIdx.x, b = blockIdx.x, gy = blockIdx.y, sp = blockIdx.z;
   const int rep = a.H / a.G, chunks = (rep + a.hpc - 1) / a.hpc;
   const int g = gy / chunks, h0 = g * rep + (gy % chunks) * a.hpc;
   const int Rc = min(a.hpc, g * rep + rep - h0);
-  const int r0 = a.blk_tab[2 * b];
-  const int nr = min(a.blk_tab[2 * b + 1], a.rows_per_blk);
+  const int r0 = a.blk_tab ? a.blk_tab[2 * b] : b;
+  const int nr = a.blk_tab ? min(a.blk_tab[2 * b + 1], a.rows_per_blk) : 1;
   const int nqv = nr * Rc;
   const int seq = a.row_seq[r0], pos0 = a.row_slot[r0], posL = pos0 + nr - 1;
   const int nbL = win_nb(posL, a.window, a.pool), tF = win_t0(pos0, a.window);
@@ -721,8 +724,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(AttnTArgs a) {
   const int ntile = (nk + KT - 1) / KT, tps = (ntile + a.nsplit - 1) / a.nsplit;
   const int t0 = sp * tps, t1 = min(ntile, t0 + tps);
   float* Kl = lds;                       // [16 keys][LDK]
-  float* Vl = Kl + KT * LDK;             // [16 keys][LDV]
-  float* Sp = Vl + KT * LDV;             // [4 waves][16 q][LDS_S] partial scores
+  float* Vl = VK ? Kl : Kl + KT * LDK;   // [16 keys][LDV]
+  float* Sp = VK ? Kl + KT * LDK : Vl + KT * LDV;   // [4 waves][16 q][LDS_S] partial scores
   float* Pl = Sp + 4 * 16 * LDS_S;       // [16 q][LDP] weights
   const int wave = tid >> 6, lane = tid & 63, c16 = lane & 15, g4 = lane >> 4;
   // the A operands of this wave's score products stay in registers for the whole key walk: query c16, values wave DQ + 4 it + g4
@@ -761,7 +764,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(AttnTArgs a) {
     const int k0 = tile * KT;
     load16<NBD>(vk, a.dim, tid, [&](int j) { const int jj = min(k0 + j, nk - 1); return jj < nbL ? pkb + (int64_t)jj * Gd : kb + (int64_t)(jj - nbL) * a.ldk; },
                 [&](int j) { return k0 + j < nk; });
-    load16<NBV>(vv, a.vdim, tid, [&](int j) { const int jj = min(k0 + j, nk - 1); return jj < nbL ? pvb + (int64_t)jj * Gv : vb + (int64_t)(jj - nbL) * a.ldv; },
+    if (!VK) load16<NBV>(vv, a.vdim, tid, [&](int j) { const int jj = min(k0 + j, nk - 1); return jj < nbL ? pvb + (int64_t)jj * Gv : vb + (int64_t)(jj - nbL) * a.ldv; },
                 [&](int j) { return k0 + j < nk; });
   };
   if (t0 < t1) fetch(t0);
@@ -769,7 +772,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(AttnTArgs a) {
     const int key0 = tile * KT;
     lds_barrier();                                             // the previous tile's keys, values and weights are consumed
     store16<NBD, LDK>(Kl, vk, tid);
-    store16<NBV, LDV>(Vl, vv, tid);
+    if (!VK) store16<NBV, LDV>(Vl, vv, tid);
     if (tile + 1 < t1) fetch(tile + 1);                          // in flight while this tile is multiplied
     lds_barrier();
     {                                                            // partial scores over this wave's quarter of the head's values
@@ -839,7 +842,9 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(AttnTArgs a) {
   }
 }
 
-// grid (n_blk, G * chunks): the splits' statistics and sums of every vector become its result
+// grid (n_blk, G * chunks, ceil(vdim / MERGE_COLS)): the splits' statistics and sums of every vector become its result; a workgroup
+// takes a slice of the value columns (one workgroup a run left the merge of a single decode row on one CU)
+constexpr int MERGE_COLS = 64;
 template <int AQ>
 __global__ __launch_bounds__(256) void window_attn_merge_kernel(AttnTArgs a) {
   const int tid = threadIdx.x, b = blockIdx.x, gy = blockIdx.y;
@@ -866,8 +871,9 @@ __global__ __launch_bounds__(256) void window_attn_merge_kernel(AttnTArgs a) {
     if (lane == 0) { Ls[i] = L; Ms[i] = mx; }
   }
   __syncthreads();
-  for (int e = tid; e < nqv * a.vdim; e += 256) {
-    const int i = e / a.vdim, c = e - i * a.vdim;
+  const int c0 = blockIdx.z * MERGE_COLS, cw = min(MERGE_COLS, a.vdim - c0);     // this workgroup's slice of the value columns
+  for (int e = tid; e < nqv * cw; e += 256) {
+    const int i = e / cw, c = c0 + e - i * cw;
     const float* src = base + 2 * AQ + (int64_t)i * a.vdim + c;
     float t = 0.f;
 #pragma unroll 4
@@ -1191,9 +1197,13 @@ AttnShape attn_shape(int H, int G, int one_row) {
 }  // namespace
 
 extern "C" int mn_window_attn_splits(int n_blk, int H, int G, int one_row, int max_keys) {
-  if (n_blk < 1 || H < 1 || G < 1 || (H % G) != 0 || max_keys < 1) return 1;
+  return mn_window_attn_splits_tile(n_blk, H, G, one_row, max_keys, AKT);
+}
+
+extern "C" int mn_window_attn_splits_tile(int n_blk, int H, int G, int one_row, int max_keys, int key_tile) {
+  if (n_blk < 1 || H < 1 || G < 1 || (H % G) != 0 || max_keys < 1 || key_tile < 1) return 1;
   const AttnShape sh = attn_shape(H, G, one_row);
-  const int64_t wgs = (int64_t)n_blk * G * sh.chunks, tiles = mn_cdiv(max_keys, AKT);
+  const int64_t wgs = (int64_t)n_blk * G * sh.chunks, tiles = mn_cdiv(max_keys, key_tile);
   int64_t ns = mn_cdiv(2 * (int64_t)mn_num_cus(), wgs);
   if (ns > tiles) ns = tiles;
   if (ns > 64) ns = 64;
@@ -1249,7 +1259,7 @@ extern "C" int mn_window_pool_attn_blocks_cap(const float* q, int64_t ldq, const
   MN_CHECK_ARG(ldk >= (int64_t)G * dim && ldv >= (int64_t)G * vdim && ((dim % 4) != 0 || (ldk % 4) == 0) && ((vdim % 4) != 0 || (ldv % 4) == 0) &&
                    softcap >= 0.0f,
                "mn_window_pool_attn_blocks: arena row strides below a row, or no multiple of 4 under heads that are; or a negative soft cap");
-  if (variant < 0) variant = (!one_row && dim <= 256 && vdim <= 256) ? MN_WINDOW_ATTN_MFMA : MN_WINDOW_ATTN_VALU;
+  const bool variant_auto = variant < 0;
   MN_CHECK_ARG(q && k_arena && v_arena && row_seq && row_slot && (out || out16) && n_blk >= 1 && H >= 1 && G >= 1 && (H % G) == 0 && dim >= 1 &&
                    vdim >= 1 && vdim <= 512 && t_max >= 1 && window >= 0 && pool >= 0 && nsplit >= 1 && nsplit <= 64,
                "mn_window_pool_attn_blocks: bad args (vdim=%d: at most 512; nsplit=%d: at most 64)", vdim, nsplit);
@@ -1261,21 +1271,42 @@ extern "C" int mn_window_pool_attn_blocks_cap(const float* q, int64_t ldq, const
                "mn_window_pool_attn_blocks: workspace too small");
   AttnTArgs a{q, ldq, k_arena, v_arena, pool ? pk : nullptr, pool ? pv : nullptr, row_seq, row_slot, one_row ? nullptr : blk_tab, H, G, dim, vdim,
               t_max, n_pool_max, window, pool, sh.rows, sh.hpc, nsplit, out_scale, out, ldo, out16, ldo16, (float*)workspace, sink, softcap, ldk, ldv};
-  MN_CHECK_ARG(variant == MN_WINDOW_ATTN_VALU || (variant == MN_WINDOW_ATTN_MFMA && !one_row && dim <= 256 && vdim <= 256),
-               "mn_window_pool_attn_blocks: the matrix-core kernel takes runs of rows with dim, vdim <= 256");
+  // values that are a view of the keys (one key/value head, the same arena and stride): the matrix-core kernel stages one tile for both
+  const bool vk = G == 1 && k_arena == v_arena && ldk == ldv && vdim <= dim && !pool;
+  const bool mfma_fits = vk ? (dim <= 640 && sh.aq == 16) : (!one_row && dim <= 256 && vdim <= 256);
+  if (variant_auto) variant = mfma_fits ? MN_WINDOW_ATTN_MFMA : MN_WINDOW_ATTN_VALU;
+  MN_CHECK_ARG(variant == MN_WINDOW_ATTN_VALU || (variant == MN_WINDOW_ATTN_MFMA && mfma_fits),
+               "mn_window_pool_attn_blocks: the matrix-core kernel takes runs of rows with dim, vdim <= 256, or values inside keys of dim <= 640");
   if (variant == MN_WINDOW_ATTN_MFMA) {
-    const int nbd = dim <= 64 ? 1 : (dim <= 128 ? 2 : 4), nbv = vdim <= 64 ? 1 : (vdim <= 128 ? 2 : 4);
-    const size_t ldsm = ((size_t)16 * (64 * nbd + 4) + (size_t)16 * (64 * nbv + 4) + 4 * 16 * 17 + 16 * 20) * sizeof(float);
     const dim3 gridm((unsigned)n_blk, (unsigned)(G * sh.chunks), (unsigned)nsplit);
     hipStream_t stm = mn_stream(stream);
+    if (vk) {
+      const int nb = dim <= 256 ? (dim + 63) / 64 : (dim <= 320 ? 5 : (dim <= 384 ? 6 : (dim <= 512 ? 8 : 10)));
+      const size_t ldsm = ((size_t)16 * (64 * nb + 4) + 4 * 16 * 17 + 16 * 20) * sizeof(float);
+#define MN_WK(D_) hipLaunchKernelGGL((window_attn_mfma_kernel<D_, D_, true>), gridm, dim3(256), ldsm, stm, a)
+      switch (nb) {
+        case 1: MN_WK(1); break;
+        case 2: MN_WK(2); break;
+        case 3: MN_WK(3); break;
+        case 4: MN_WK(4); break;
+        case 5: MN_WK(5); break;
+        case 6: MN_WK(6); break;
+        case 8: MN_WK(8); break;
+        default: MN_WK(10); break;
+      }
+#undef MN_WK
+    } else {
+      const int nbd = dim <= 64 ? 1 : (dim <= 128 ? 2 : 4), nbv = vdim <= 64 ? 1 : (vdim <= 128 ? 2 : 4);
+      const size_t ldsm = ((size_t)16 * (64 * nbd + 4) + (size_t)16 * (64 * nbv + 4) + 4 * 16 * 17 + 16 * 20) * sizeof(float);
 #define MN_WM(D_, V_) hipLaunchKernelGGL((window_attn_mfma_kernel<D_, V_>), gridm, dim3(256), ldsm, stm, a)
-    if (nbd == 1) { if (nbv == 1) MN_WM(1, 1); else if (nbv == 2) MN_WM(1, 2); else MN_WM(1, 4); }
-    else if (nbd == 2) { if (nbv == 1) MN_WM(2, 1); else if (nbv == 2) MN_WM(2, 2); else MN_WM(2, 4); }
-    else { if (nbv == 1) MN_WM(4, 1); else if (nbv == 2) MN_WM(4, 2); else MN_WM(4, 4); }
+      if (nbd == 1) { if (nbv == 1) MN_WM(1, 1); else if (nbv == 2) MN_WM(1, 2); else MN_WM(1, 4); }
+      else if (nbd == 2) { if (nbv == 1) MN_WM(2, 1); else if (nbv == 2) MN_WM(2, 2); else MN_WM(2, 4); }
+      else { if (nbv == 1) MN_WM(4, 1); else if (nbv == 2) MN_WM(4, 2); else MN_WM(4, 4); }
 #undef MN_WM
+    }
     MN_CHECK_LAUNCH("mn_window_pool_attn_blocks(mfma)");
     if (nsplit > 1) {
-      hipLaunchKernelGGL((window_attn_merge_kernel<16>), dim3((unsigned)n_blk, (unsigned)(G * sh.chunks)), dim3(256), 0, stm, a);
+      hipLaunchKernelGGL((window_attn_merge_kernel<16>), dim3((unsigned)n_blk, (unsigned)(G * sh.chunks), (unsigned)mn_cdiv(vdim, MERGE_COLS)), dim3(256), 0, stm, a);
       MN_CHECK_LAUNCH("mn_window_pool_attn_blocks(merge)");
     }
     return MN_OK;
@@ -1294,7 +1325,7 @@ extern "C" int mn_window_pool_attn_blocks_cap(const float* q, int64_t ldq, const
   }
   MN_CHECK_LAUNCH("mn_window_pool_attn_blocks");
   if (nsplit > 1) {
-    const dim3 mg((unsigned)n_blk, (unsigned)(G * sh.chunks));
+    const dim3 mg((unsigned)n_blk, (unsigned)(G * sh.chunks), (unsigned)mn_cdiv(vdim, MERGE_COLS));
     if (sh.aq == 4) hipLaunchKernelGGL((window_attn_merge_kernel<4>), mg, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((window_attn_merge_kernel<16>), mg, dim3(256), 0, st, a);
     MN_CHECK_LAUNCH("mn_window_pool_attn_blocks(merge)");

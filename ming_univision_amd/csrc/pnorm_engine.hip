@@ -184,7 +184,8 @@ extern "C" int mn_pn_step(const mn_pn_model* m, const mn_pn_state* st, const flo
       }
       int keys = max_len;
       if (l.window > 0 && l.window + 3 < keys) keys = l.window + 3;
-      int ns = mn_window_attn_splits(n_blk, H, G, one_row, keys);
+      // latent attention's decode rows run on the matrix-core kernel (all heads of a row in one workgroup): its key tiles hold 16 keys
+      int ns = mn_window_attn_splits_tile(n_blk, H, G, one_row, keys, latent && one_row ? 16 : 64);
       while (ns > 1 && mn_window_attn_workspace_bytes(n_blk, H, G, d.avd, one_row, ns) > p.attn_ws) --ns;
       const bool gate = attn && l.has_gate;
       MN_TRY(mn_window_pool_attn_blocks_cap(qf, d.nq, karena, ldk, varena, ldv, nullptr, nullptr, nullptr, l.softcap, row_seq, row_slot, blk_tab,

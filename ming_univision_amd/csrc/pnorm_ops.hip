@@ -11,6 +11,7 @@
 #include <math.h>
 
 #include "common.h"
+#include "mfma_f32_tiles.h"
 
 extern "C" int mn_rotary_frequencies_scaled_host(int dims, double base, double factor, double low, double high, double original, float* freq) {
   MN_CHECK_ARG(freq && dims >= 2 && (dims % 2) == 0 && base > 0.0 && factor >= 0.0, "mn_rotary_frequencies_scaled_host: bad args");
@@ -249,15 +250,26 @@ __device__ __forceinline__ float sum8(float v) {                    // over the 
 
 // Rows of sequences (a prompt portion): grid (M, H, ceil(vdim / 32)); the workgroup of a sequence's FIRST row in the call walks that
 // sequence's rows.  A workgroup owns 32 value columns; 8 lanes share a column, lane s of them holds the state rows s, s + 8, ... in
-// registers (NR of them; NR = 0: the column stays in the arena, any dim).  q and k of the next row are loaded while the current row
-// is computed and staged through LDS (two buffers, one barrier per row).
+// registers (NR of them; NR = 0: the column stays in the arena, any dim).  The rows are taken in batches of DB: a batch's q, k, v,
+// write strengths and decays go global -> registers (while the previous batch is computed) -> LDS, k . q of every row is summed once
+// per workgroup, and the DB steps of the recurrence then run from LDS and registers alone — a step is two partial dot products, one
+// reduction over the 8 lanes and the update, with no barrier and no memory latency between steps.
+constexpr int DB = 16;
 template <int NR>
 __global__ __launch_bounds__(256) void delta_rows_kernel(DeltaArgs a) {
-  extern __shared__ float lds[];             // [2][2 dim]
-  const int m0 = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, s = tid & 7, c = blockIdx.z * 32 + (tid >> 3);
+  extern __shared__ float lds[];             // [DB][2 dim] q, k; [DB][32] v; [DB] beta, decay, k . q
+  const int m0 = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, s = tid & 7, cl = tid >> 3, c = blockIdx.z * 32 + cl;
   if (a.row_back[m0] != 0) return;
   const int d = a.dim, kvh = h / (a.H / a.G);
   const bool on = c < a.vdim;
+  // rows of this sequence in the call: they are consecutive, so the rows that continue it form a prefix of every 256 looked at
+  int n = 1;
+  for (;;) {
+    const int m = m0 + n + tid;
+    const int cnt = __syncthreads_count(m < a.M && a.row_back[m] == m - m0);
+    n += cnt;
+    if (cnt < 256) break;
+  }
   float* sp = a.state + (((int64_t)a.row_seq[m0] * a.H + h) * d) * a.vdim + (on ? c : 0);
   const bool fresh = a.row_slot[m0] == 0;
   constexpr int NS = NR > 0 ? NR : 1;
@@ -268,58 +280,208 @@ __global__ __launch_bounds__(256) void delta_rows_kernel(DeltaArgs a) {
   } else if (fresh && on) {
     for (int i = s; i < d; i += 8) sp[(int64_t)i * a.vdim] = 0.f;
   }
-  constexpr int NST = 4;                      // staged values per thread: 2 dim <= 1024
-  auto src_of = [&](int m, int i) { return a.qkv + (int64_t)m * a.ld + (i < d ? 0 : a.G * d) + (int64_t)kvh * d + (i < d ? i : i - d); };
-  float stg[NST];
+  float* qk = lds;                           // row r: q at r * 2 d, k at r * 2 d + d
+  float* vs = qk + DB * 2 * d;               // [DB][32]
+  float* bs = vs + DB * 32;                  // [DB] beta, [DB] decay, [DB] k . q
+  constexpr int NQ = 32;                     // staged q / k values per thread and batch: DB * 2 dim / 256 <= 32 for dim <= 256
+  const int per = 2 * d * DB;
+  float rq[NQ], rv[2], rb = 0.f;
+  auto fetch = [&](int b0) {                 // batch rows b0 .. b0 + DB of the sequence into registers
+    const int rows = min(DB, n - b0);
 #pragma unroll
-  for (int t = 0; t < NST; ++t) { const int i = tid + 256 * t; if (i < 2 * d) lds[i] = *src_of(m0, i); }
-  float v = on ? a.qkv[(int64_t)m0 * a.ld + 2 * a.G * d + (int64_t)h * a.vdim + c] : 0.f;
-  float beta = a.bd[(int64_t)m0 * a.ldbd + h], g = a.bd[(int64_t)m0 * a.ldbd + a.H + h];
-  int buf = 0;
-  for (int m = m0;; ++m, buf ^= 1) {
+    for (int t = 0; t < NQ; ++t) {
+      const int e = tid + 256 * t;
+      if (e < per) {
+        const int r = e / (2 * d), i = e - r * 2 * d;
+        rq[t] = r < rows ? a.qkv[(int64_t)(m0 + b0 + r) * a.ld + (i < d ? 0 : a.G * d) + (int64_t)kvh * d + (i < d ? i : i - d)] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int e = tid + 256 * t, r = e >> 5, cc = blockIdx.z * 32 + (e & 31);
+      rv[t] = (r < rows && cc < a.vdim) ? a.qkv[(int64_t)(m0 + b0 + r) * a.ld + 2 * a.G * d + (int64_t)h * a.vdim + cc] : 0.f;
+    }
+    if (tid < 2 * DB) {
+      const int r = tid % DB;
+      rb = r < rows ? a.bd[(int64_t)(m0 + b0 + r) * a.ldbd + (tid < DB ? 0 : a.H) + h] : 0.f;
+    }
+  };
+  fetch(0);
+  for (int b0 = 0; b0 < n; b0 += DB) {
+    const int rows = min(DB, n - b0);
+    __syncthreads();                         // the previous batch's steps have read their rows
+    if (NR > 0 || d <= 256) {
+#pragma unroll
+      for (int t = 0; t < NQ; ++t) { const int e = tid + 256 * t; if (e < per) qk[e] = rq[t]; }
+    } else {                                 // larger heads than the registers stage: straight from memory
+      for (int e = tid; e < per; e += 256) {
+        const int r = e / (2 * d), i = e - r * 2 * d;
+        qk[e] = r < rows ? a.qkv[(int64_t)(m0 + b0 + r) * a.ld + (i < d ? 0 : a.G * d) + (int64_t)kvh * d + (i < d ? i : i - d)] : 0.f;
+      }
+    }
+    vs[tid] = rv[0]; vs[tid + 256] = rv[1];
+    if (tid < 2 * DB) bs[tid] = rb;
     __syncthreads();
-    const bool more = m + 1 < a.M && a.row_back[m + 1] == m + 1 - m0;
-    float nv = 0.f, nbeta = 0.f, ng = 0.f;
-    if (more) {
-#pragma unroll
-      for (int t = 0; t < NST; ++t) { const int i = tid + 256 * t; if (i < 2 * d) stg[t] = *src_of(m + 1, i); }
-      nv = on ? a.qkv[(int64_t)(m + 1) * a.ld + 2 * a.G * d + (int64_t)h * a.vdim + c] : 0.f;
-      nbeta = a.bd[(int64_t)(m + 1) * a.ldbd + h];
-      ng = a.bd[(int64_t)(m + 1) * a.ldbd + a.H + h];
+    if (b0 + DB < n) fetch(b0 + DB);         // in flight while this batch is computed
+    {                                        // k . q of every row: 16 threads a row
+      const int r = tid >> 4, l = tid & 15;
+      float t = 0.f;
+      for (int i = l; i < d; i += 16) t = fmaf(qk[r * 2 * d + i], qk[r * 2 * d + d + i], t);
+      t = row16_sum(t);
+      if (l == 0) bs[2 * DB + r] = t;
     }
-    const float* q = lds + buf * 2 * d;
-    const float* k = q + d;
-    float pk = 0.f, pq = 0.f, kq = 0.f;
-    if (NR > 0) {
+    lds_barrier();                           // orders LDS only: the next batch's loads stay in flight
+    for (int r = 0; r < rows; ++r) {
+      const float* q = qk + r * 2 * d;
+      const float* k = q + d;
+      const float v = vs[r * 32 + cl], beta = bs[r], g = bs[DB + r], kq = bs[2 * DB + r];
+      float pk = 0.f, pq = 0.f;
+      if (NR > 0) {
 #pragma unroll
-      for (int j = 0; j < NS; ++j) {
-        const int i = s + 8 * j;
-        if (i < d) { const float kk = k[i], qq = q[i]; pk = fmaf(S[j], kk, pk); pq = fmaf(S[j], qq, pq); kq = fmaf(kk, qq, kq); }
+        for (int j = 0; j < NS; ++j) {
+          const int i = s + 8 * j;
+          if (i < d) { pk = fmaf(S[j], k[i], pk); pq = fmaf(S[j], q[i], pq); }
+        }
+      } else {
+        for (int i = s; i < d; i += 8) {
+          const float sv = on ? sp[(int64_t)i * a.vdim] : 0.f;
+          pk = fmaf(sv, k[i], pk); pq = fmaf(sv, q[i], pq);
+        }
       }
-    } else {
-      for (int i = s; i < d; i += 8) {
-        const float sv = on ? sp[(int64_t)i * a.vdim] : 0.f, kk = k[i], qq = q[i];
-        pk = fmaf(sv, kk, pk); pq = fmaf(sv, qq, pq); kq = fmaf(kk, qq, kq);
+      pk = sum8(pk); pq = sum8(pq);
+      const float u = beta * (v - g * pk);
+      if (NR > 0) {
+#pragma unroll
+        for (int j = 0; j < NS; ++j) { const int i = s + 8 * j; if (i < d) S[j] = fmaf(g, S[j], k[i] * u); }
+      } else if (on) {
+        for (int i = s; i < d; i += 8) sp[(int64_t)i * a.vdim] = fmaf(g, sp[(int64_t)i * a.vdim], k[i] * u);
       }
+      if (on && s == 0) a.out[(int64_t)(m0 + b0 + r) * a.ldo + (int64_t)h * a.vdim + c] = fmaf(g, pq, u * kq);
     }
-    pk = sum8(pk); pq = sum8(pq); kq = sum8(kq);
-    const float u = beta * (v - g * pk);
-    if (NR > 0) {
-#pragma unroll
-      for (int j = 0; j < NS; ++j) { const int i = s + 8 * j; if (i < d) S[j] = fmaf(g, S[j], k[i] * u); }
-    } else if (on) {
-      for (int i = s; i < d; i += 8) sp[(int64_t)i * a.vdim] = fmaf(g, sp[(int64_t)i * a.vdim], k[i] * u);
-    }
-    if (on && s == 0) a.out[(int64_t)m * a.ldo + (int64_t)h * a.vdim + c] = fmaf(g, pq, u * kq);
-    if (!more) break;
-    float* nx = lds + (buf ^ 1) * 2 * d;
-#pragma unroll
-    for (int t = 0; t < NST; ++t) { const int i = tid + 256 * t; if (i < 2 * d) nx[i] = stg[t]; }
-    v = nv; beta = nbeta; g = ng;
   }
   if (NR > 0 && on) {
 #pragma unroll
     for (int j = 0; j < NS; ++j) { const int i = s + 8 * j; if (i < d) sp[(int64_t)i * a.vdim] = S[j]; }
+  }
+}
+
+// The same walk for heads of at most 256 state rows, without a branch in the step: grid (H * ceil(vdim / CPB), M) — the workgroups that
+// work (those of a sequence's first row) are neighbours in the launch order and land on different CUs.  LPC lanes share a value column
+// (CPB = 256 / LPC columns a workgroup); a lane holds the state rows 4 (s + LPC jj) + t, t < 4, jj < NS / 4, so that q and k come from
+// LDS in 16-byte reads; LDS rows are padded with zeros to DP = NS * LPC values, under which the padded state rows stay zero.
+template <int NS, int LPC, int DBT>
+__global__ __launch_bounds__(256) void delta_rows_fast_kernel(DeltaArgs a) {
+  constexpr int CPB = 256 / LPC, DP = NS * LPC, NQ = DBT * 2 * DP / 256, NV = (DBT * CPB + 255) / 256;
+  extern __shared__ float lds[];             // [DBT][2 DP] q, k; [DBT][CPB] v; [DBT] beta, decay, k . q; [DBT][CPB] outputs
+  const int m0 = blockIdx.y, ncb = (a.vdim + CPB - 1) / CPB, h = blockIdx.x / ncb, cb = blockIdx.x - h * ncb;
+  const int tid = threadIdx.x, s = tid % LPC, cl = tid / LPC, c = cb * CPB + cl;
+  if (a.row_back[m0] != 0) return;
+  const int d = a.dim, kvh = h / (a.H / a.G);
+  const bool on = c < a.vdim;
+  int n = 1;
+  for (;;) {
+    const int m = m0 + n + tid;
+    const int cnt = __syncthreads_count(m < a.M && a.row_back[m] == m - m0);
+    n += cnt;
+    if (cnt < 256) break;
+  }
+  float* sp = a.state + (((int64_t)a.row_seq[m0] * a.H + h) * d) * a.vdim + (on ? c : 0);
+  const bool fresh = a.row_slot[m0] == 0;
+  float S[NS];
+#pragma unroll
+  for (int j = 0; j < NS; ++j) {
+    const int i = 4 * (s + LPC * (j >> 2)) + (j & 3);
+    S[j] = (on && !fresh && i < d) ? sp[(int64_t)i * a.vdim] : 0.f;
+  }
+  float* qk = lds;                           // row r: q at r * 2 DP, k at r * 2 DP + DP
+  float* vs = qk + DBT * 2 * DP;
+  float* bs = vs + DBT * CPB;
+  float* os = bs + 3 * DBT;                   // [DBT][CPB] the batch's outputs
+  float rq[NQ], rv[NV], rb = 0.f;
+  // element e of a batch's q / k block: row e / (2 DP), value e % (2 DP) (q below DP, k from DP on)
+  auto fetch = [&](int b0) {
+    const int rows = min(DBT, n - b0);
+#pragma unroll
+    for (int t = 0; t < NQ; ++t) {
+      const int e = tid + 256 * t, r = e / (2 * DP), i = e % (2 * DP), ii = i % DP;
+      rq[t] = (r < rows && ii < d) ? a.qkv[(int64_t)(m0 + b0 + r) * a.ld + (i < DP ? 0 : a.G * d) + (int64_t)kvh * d + ii] : 0.f;
+    }
+#pragma unroll
+    for (int t = 0; t < NV; ++t) {
+      const int e = tid + 256 * t, r = e / CPB, cc = cb * CPB + e % CPB;
+      rv[t] = (r < rows && cc < a.vdim) ? a.qkv[(int64_t)(m0 + b0 + r) * a.ld + 2 * a.G * d + (int64_t)h * a.vdim + cc] : 0.f;
+    }
+    if (tid < 2 * DBT) {
+      const int r = tid % DBT;
+      rb = r < rows ? a.bd[(int64_t)(m0 + b0 + r) * a.ldbd + (tid < DBT ? 0 : a.H) + h] : 0.f;
+    }
+  };
+  fetch(0);
+  for (int b0 = 0; b0 < n; b0 += DBT) {
+    const int rows = min(DBT, n - b0);
+    lds_barrier();                           // the previous batch's steps have read their rows
+#pragma unroll
+    for (int t = 0; t < NQ; ++t) qk[tid + 256 * t] = rq[t];
+#pragma unroll
+    for (int t = 0; t < NV; ++t) { const int e = tid + 256 * t; if (e < DBT * CPB) vs[e] = rv[t]; }
+    if (tid < 2 * DBT) bs[tid] = rb;
+    lds_barrier();
+    if (b0 + DBT < n) fetch(b0 + DBT);         // in flight while this batch is computed
+    for (int r = tid >> 4; r < DBT; r += 16) {   // k . q of every row: 16 threads a row
+      const int l = tid & 15;
+      float t = 0.f;
+#pragma unroll
+      for (int i = l; i < DP; i += 16) t = fmaf(qk[r * 2 * DP + i], qk[r * 2 * DP + DP + i], t);
+      t = row16_sum(t);
+      if (l == 0) bs[2 * DBT + r] = t;
+    }
+    lds_barrier();                           // orders LDS only: the next batch's loads stay in flight
+    // the operands of step r + 1 are read from LDS before step r is computed: they do not depend on the state
+    float kk[NS], qq[NS], v, beta, g, kq;
+    auto load_row = [&](int r, float (&k_)[NS], float (&q_)[NS], float& v_, float& b_, float& g_, float& kq_) {
+      const float* q = qk + r * 2 * DP + 4 * s;
+#pragma unroll
+      for (int jj = 0; jj < NS / 4; ++jj) {
+        const float4 k4 = *reinterpret_cast<const float4*>(q + DP + 4 * LPC * jj), q4 = *reinterpret_cast<const float4*>(q + 4 * LPC * jj);
+        k_[4 * jj] = k4.x; k_[4 * jj + 1] = k4.y; k_[4 * jj + 2] = k4.z; k_[4 * jj + 3] = k4.w;
+        q_[4 * jj] = q4.x; q_[4 * jj + 1] = q4.y; q_[4 * jj + 2] = q4.z; q_[4 * jj + 3] = q4.w;
+      }
+      v_ = vs[r * CPB + cl]; b_ = bs[r]; g_ = bs[DBT + r]; kq_ = bs[2 * DBT + r];
+    };
+    load_row(0, kk, qq, v, beta, g, kq);
+#pragma unroll 2
+    for (int r = 0; r < rows; ++r) {
+      float kn[NS], qn[NS], vn, bn, gn, kqn;
+      load_row(min(r + 1, DBT - 1), kn, qn, vn, bn, gn, kqn);
+      float pk = 0.f, pq = 0.f, pk2 = 0.f, pq2 = 0.f;
+#pragma unroll
+      for (int j = 0; j < NS; j += 2) {
+        pk = fmaf(S[j], kk[j], pk); pk2 = fmaf(S[j + 1], kk[j + 1], pk2);
+        pq = fmaf(S[j], qq[j], pq); pq2 = fmaf(S[j + 1], qq[j + 1], pq2);
+      }
+      pk += pk2; pq += pq2;
+      if (LPC == 16) { pk = row16_sum(pk); pq = row16_sum(pq); } else { pk = sum8(pk); pq = sum8(pq); }
+      const float u = beta * (v - g * pk);
+#pragma unroll
+      for (int j = 0; j < NS; ++j) S[j] = fmaf(g, S[j], kk[j] * u);
+      if (s == 0) os[r * CPB + cl] = fmaf(g, pq, u * kq);
+#pragma unroll
+      for (int j = 0; j < NS; ++j) { kk[j] = kn[j]; qq[j] = qn[j]; }
+      v = vn; beta = bn; g = gn; kq = kqn;
+    }
+    lds_barrier();
+#pragma unroll
+    for (int t = 0; t < NV; ++t) {           // the batch's outputs, a row's columns side by side
+      const int e = tid + 256 * t, r = e / CPB, cc = cb * CPB + e % CPB;
+      if (r < rows && cc < a.vdim) a.out[(int64_t)(m0 + b0 + r) * a.ldo + (int64_t)h * a.vdim + cc] = os[e];
+    }
+  }
+  if (on) {
+#pragma unroll
+    for (int j = 0; j < NS; ++j) {
+      const int i = 4 * (s + LPC * (j >> 2)) + (j & 3);
+      if (i < d) sp[(int64_t)i * a.vdim] = S[j];
+    }
   }
 }
 
@@ -472,12 +634,21 @@ extern "C" int mn_gated_delta_rows(const float* qkv, int64_t ld, const float* bd
     MN_CHECK_LAUNCH("mn_gated_delta_rows(step)");
     return MN_OK;
   }
-  const size_t lds = (size_t)4 * dim * sizeof(float);
-  if (dim <= 32) hipLaunchKernelGGL((delta_rows_kernel<4>), grid, dim3(256), lds, st, a);
-  else if (dim <= 64) hipLaunchKernelGGL((delta_rows_kernel<8>), grid, dim3(256), lds, st, a);
-  else if (dim <= 128) hipLaunchKernelGGL((delta_rows_kernel<16>), grid, dim3(256), lds, st, a);
-  else if (dim <= 256) hipLaunchKernelGGL((delta_rows_kernel<32>), grid, dim3(256), lds, st, a);
-  else hipLaunchKernelGGL((delta_rows_kernel<0>), grid, dim3(256), lds, st, a);
+  if (dim <= 256) {
+    MN_CHECK_ARG(M <= 65535 && (int64_t)H * mn_cdiv(vdim, 16) < ((int64_t)1 << 31), "mn_gated_delta_rows: too many rows or columns");
+#define MN_DF(NS_, LPC_, DB_)                                                                                                                 \
+  hipLaunchKernelGGL((delta_rows_fast_kernel<NS_, LPC_, DB_>), dim3((unsigned)(H * mn_cdiv(vdim, 256 / LPC_)), (unsigned)M), dim3(256),  \
+                     ((size_t)DB_ * 2 * NS_ * LPC_ + 2 * DB_ * (256 / LPC_) + 3 * DB_) * sizeof(float), st, a)
+    if (dim <= 32) MN_DF(4, 8, 32); else if (dim <= 64) MN_DF(4, 16, 32); else if (dim <= 128) MN_DF(8, 16, 32); else MN_DF(16, 16, 16);
+#undef MN_DF
+  } else {
+    const size_t lds = ((size_t)DB * 2 * dim + DB * 32 + 3 * DB) * sizeof(float);    // 16 rows of q and k: 64 KiB at dim 512
+    if (lds > 64 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&delta_rows_kernel<0>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      MN_CHECK_ARG(e == hipSuccess, "mn_gated_delta_rows: %zu bytes of LDS refused (dim=%d)", lds, dim);
+    }
+    hipLaunchKernelGGL((delta_rows_kernel<0>), grid, dim3(256), lds, st, a);
+  }
   MN_CHECK_LAUNCH("mn_gated_delta_rows");
   return MN_OK;
 }

@@ -1,5 +1,5 @@
 """Prefill / decode throughput of the Pizitar, the Sakinex or the Zuzenex decoder beside the Bailing-MoE decoder at equal size
-(`bench.py --lm-compare [--lm-model sakinex | zuzenex]`).
+(`bench.py --lm-compare [--lm-model sakinex | zuzenex]`), and of the Daberax decoder beside the Zuzenex decoder (`--lm-model daberax`).
 
 Random weights at sizes that resemble real layers.  "Equal size": same width, depth and head count, 128-wide heads on both, and a
 feed-forward whose ACTIVE hidden width matches (the MoE runs 8 experts, top-2, of half the dense hidden width each).  Both run
@@ -22,6 +22,13 @@ have three, so they are 1.5 times as wide: the same parameters per expert).  Its
 decoder's, and is priced the same way — on the fp32 matrix-core peak for prompts (its scores and weights are 32-bit) and on the cache
 bytes for decode rows; the recurrence alone is priced on its multiply-adds (prompts: the chunked scan) and on the state bytes it reads
 and writes (decode rows).
+
+Daberax stands beside Zuzenex, the closest model of the framework (both choose attention or a matrix-state recurrence per layer): same
+width, depth, head counts and 128-wide heads, dense feed-forwards of equal parameter count on both (three matrices of width ff against
+two of 1.5 ff), layers latent - delta - delta - attention against attention - lightning - lightning - attention.  Daberax's attentions
+see a window of 1024 tokens and are priced on the keys they see; its latent attention reads [latent ; rotated part] once per key (the
+values are a view of the keys); the delta rule is priced like the lightning recurrence — prompts on the multiply-adds of the recurrence
+(three products of a dim x vdim state per token and head), decode rows on the state bytes read and written.
 """
 import time
 
@@ -220,22 +227,24 @@ def run_sakinex(s, T, batches, n_dec):
     return out
 
 
-def zuzenex_config(s):
+def zuzenex_config(s, dense=False):
     from .configuration import ZuzenexConfig
     H = s["heads"]
     mlp = dict(kind="moe", router=dict(experts=8, top=2, identity=1), expert=dict(ff=s["ff"] * 3 // 4), shared=dict(ff=s["ff"] * 3 // 4))
+    if dense:
+        mlp = dict(kind="dense", ff=s["ff"] * 3 // 2)
     att = dict(type="attention", mixer=dict(heads=H, kv_heads=H // 4, dim=128, vdim=128, scale=128 ** -0.5, q_temp=dict(coef=0.1, every=1024)), mlp=mlp)
     lin = dict(type="lightning", mixer=dict(heads=H, dim=128, vdim=128, decay=[1.0 - 2.0 ** (-5 - 4 * h / H) for h in range(H)]), mlp=mlp)
     order = [att, lin, lin, att]
     return ZuzenexConfig(width=s["width"], vocab=s["vocab"], layers=[order[i % 4] for i in range(s["layers"])], norm=dict(eps=1e-6))
 
 
-def run_zuzenex(s, T, batches, n_dec):
+def run_zuzenex(s, T, batches, n_dec, dense=False):
     from ._lib import check, current_stream, lib, ptr
     from .sequences import rows_of_spans
     from .zuzenex import ZuzenexDecoder
     dev = "cuda"
-    cfg = zuzenex_config(s)
+    cfg = zuzenex_config(s, dense)
     dec = ZuzenexDecoder.synthetic(cfg, dev, t_max=T + n_dec + 8, n_seq=max(batches), arith="bf16")
     ids = torch.randint(0, s["vocab"], (T,), device=dev)
     x = dec.embed(ids)
@@ -315,6 +324,116 @@ def run_zuzenex(s, T, batches, n_dec):
     return out
 
 
+def daberax_config(s, window=1024):
+    from .configuration import DaberaxConfig
+    H = s["heads"]
+    mlp = dict(kind="dense", ff=s["ff"])
+    att = dict(type="attention", mixer=dict(heads=H, kv_heads=H // 4, dim=128, vdim=128, scale=128 ** -0.5, softcap=30.0, mask=dict(size=window),
+                                            rot=dict(base=500000.0, dims=128, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))), mlp=mlp)
+    lat = dict(type="latent_attention", mixer=dict(heads=H, dim=128, rot_dim=64, vdim=128, kv_rank=s["kv_rank"], scale=192 ** -0.5,
+                                                   mask=dict(size=window), rot=dict(base=10000.0, dims=64)), mlp=mlp)
+    dlt = dict(type="delta", mixer=dict(heads=H, kv_heads=H // 2, dim=128, vdim=128, conv=4), mlp=mlp)
+    order = [lat, dlt, dlt, att]
+    return DaberaxConfig(width=s["width"], vocab=s["vocab"], layers=[order[i % 4] for i in range(s["layers"])], norm=dict(eps=1e-6),
+                         token_side=dict(dim=64), logit_scale=0.5)
+
+
+def run_daberax(s, T, batches, n_dec, window=1024):
+    from ._lib import check, current_stream, lib, ptr
+    from .daberax import DaberaxDecoder
+    from .sequences import rows_of_spans
+    dev = "cuda"
+    cfg = daberax_config(s, window)
+    dec = DaberaxDecoder.synthetic(cfg, dev, t_max=T + n_dec + 8, n_seq=max(batches), arith="bf16")
+    ids = torch.randint(0, s["vocab"], (T,), device=dev)
+    x = dec.embed(ids)
+    out = {"prefill_tokens_per_s": T / _time(lambda: dec.forward_spans(x, [(0, T, 0)], tokens=ids), 3)}
+    for B in batches:
+        for ly in dec.state_t:                               # every sequence continues the prompt of sequence 0
+            for t in ly.values():
+                if t is not None and B > 1:
+                    t[1:B].copy_(t[0:1].expand_as(t[1:B]))
+        row_seq = torch.arange(B, dtype=torch.int32, device=dev)
+        back, blk = dec.decode_tables(B)
+        tok = torch.randint(0, s["vocab"], (B,), device=dev)
+        xb, tok32 = dec.embed(tok), tok.to(torch.int32)
+
+        def loop():
+            slot = torch.full((B,), T, dtype=torch.int32, device=dev)
+            ln = slot + 1
+            for i in range(n_dec):
+                dec.step(xb, row_seq, slot, back, ln, blk, T + i + 1, distinct=True, row_tok=tok32)
+                check(lib().mn_rows_advance(ptr(slot), ptr(ln), None, B, 1, current_stream()), "mn_rows_advance")
+        out[f"decode_b{B}_tokens_per_s"] = B * n_dec / _time(loop, 2, 1)
+        slot_g = torch.full((B,), T, dtype=torch.int32, device=dev)
+        ln_g = slot_g + 1
+        graph = dec.decode_graph(row_seq, slot_g, ln_g)
+
+        def loop_graph():
+            slot_g.fill_(T)
+            ln_g.fill_(T + 1)
+            for i in range(n_dec):
+                graph.run(xb, T + i + 1, tokens=tok32)
+        out[f"decode_b{B}_graph_tokens_per_s"] = B * n_dec / _time(loop_graph, 2, 1)
+    # the kernels alone, on the layers' own arenas and states
+    H = s["heads"]
+    RB = lib().mn_window_attn_block_rows()
+    tabs = {k: torch.from_numpy(v).to(dev) for k, v in rows_of_spans([(0, T, 0)], RB).items() if k != "max_len"}
+    aws = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+    pairs = sum(min(i + 1, window) for i in range(T))       # (query, key) pairs a prompt of T rows sees
+    seen = min(T, window)
+
+    def attention(name, li, G, dk, dv, ldk, v_of_k):
+        st = dec.state_t[li]
+        q = torch.randn(T, H * dk, device=dev) * 0.05
+        att = torch.empty(T, H * dv, device=dev)
+        varena = st["k"] if v_of_k else st["v"]
+
+        def attn(M, rs, rp, one_row):
+            n_blk = M if one_row else tabs["blk_tab"].shape[0]
+            ns = lib().mn_window_attn_splits_tile(n_blk, H, G, one_row, seen, 16 if (v_of_k and one_row) else 64)
+            check(lib().mn_window_pool_attn_blocks_cap(ptr(q), H * dk, ptr(st["k"]), ldk, ptr(varena), ldk if v_of_k else 0, None, None, None, 30.0,
+                                                       ptr(rs), ptr(rp), None if one_row else ptr(tabs["blk_tab"]), n_blk, one_row, H, G, dk, dv,
+                                                       dec.t_max, 1, window, 0, 1.0, ptr(att), H * dv, None, 0, ns, ptr(aws), aws.numel(), -1,
+                                                       current_stream()), "mn_window_pool_attn_blocks_cap")
+            return ns
+        t = _time(lambda: attn(T, tabs["row_seq"], tabs["row_slot"], 0), 5)
+        flops = 2 * H * (dk + dv) * pairs
+        out[name + "_prefill"] = dict(us=t * 1e6, tflops=flops / t / 1e12, of_peak=flops / t / 1e12 / FMA_F32_TFLOPS,
+                                      peak="fp32 MFMA" if max(dk, dv) <= 256 else "fp32 FMA")
+        for B in batches:
+            row_seq = torch.arange(B, dtype=torch.int32, device=dev)
+            slot = torch.full((B,), T - 1, dtype=torch.int32, device=dev)
+            t = _time(lambda: attn(B, row_seq, slot, 1), 20)
+            byts = B * seen * (ldk if v_of_k else G * (dk + dv)) * 4
+            out[f"{name}_decode_b{B}"] = dict(us=t * 1e6, gbs=byts / t / 1e9, of_peak=byts / t / 1e9 / HBM_GBS, key_splits=attn(B, row_seq, slot, 1))
+    R = s["kv_rank"]
+    attention("latent_attn", 0, 1, R + 64, R, lib().mn_pn_latent_ld(R, 64), True)
+    attention("attn", 3, H // 4, 128, 128, 0, False)
+    # the delta rule alone, on the second layer's state
+    d, G = 128, H // 2
+    lin = dec.state_t[1]["lin"]
+    qkv = torch.randn(T, 2 * G * d + H * d, device=dev)
+    qkv[:, :2 * G * d] *= d ** -0.5
+    bd = torch.cat([torch.rand(T, H, device=dev), 0.9 + 0.1 * torch.rand(T, H, device=dev)], 1).contiguous()
+    o = torch.empty(T, H * d, device=dev)
+
+    def delta(M, rs, rp, rb, flags):
+        check(lib().mn_gated_delta_rows(ptr(qkv), qkv.shape[1], ptr(bd), 2 * H, M, H, G, d, d, ptr(lin), ptr(rs), ptr(rp), ptr(rb), flags, ptr(o),
+                                        H * d, current_stream()), "mn_gated_delta_rows")
+    t = _time(lambda: delta(T, tabs["row_seq"], tabs["row_slot"], tabs["row_back"], 0), 5)
+    flops = 2 * T * H * 3 * d * d
+    out["delta_prefill"] = dict(us=t * 1e6, tflops=flops / t / 1e12, of_peak=flops / t / 1e12 / FMA_F32_TFLOPS, peak="fp32 FMA")
+    for B in batches:
+        row_seq = torch.arange(B, dtype=torch.int32, device=dev)
+        slot = torch.full((B,), T - 1, dtype=torch.int32, device=dev)
+        back = torch.zeros(B, dtype=torch.int32, device=dev)
+        t = _time(lambda: delta(B, row_seq, slot, back, 1), 20)
+        byts = B * H * d * d * 4 * 2
+        out[f"delta_decode_b{B}"] = dict(us=t * 1e6, gbs=byts / t / 1e9, of_peak=byts / t / 1e9 / HBM_GBS)
+    return out
+
+
 def run_bailing(s, T, batches, n_dec, shared=0):
     from . import ops
     from ._lib import check, current_stream, lib, ptr
@@ -364,6 +483,11 @@ def compare(sizes=("w1024", "w2048"), prompt=2048, batches=(1, 32), n_dec=32, mo
     for name in sizes:
         s = SIZES[name]
         torch.cuda.empty_cache()
+        if model == "daberax":                               # beside the closest model of the framework instead of the Bailing-MoE decoder
+            res[name] = dict(size=s, prompt=prompt, daberax=run_daberax(s, prompt, batches, n_dec))
+            torch.cuda.empty_cache()
+            res[name]["zuzenex_dense"] = run_zuzenex(s, prompt, batches, n_dec, dense=True)
+            continue
         if model == "zuzenex":
             res[name] = dict(size=s, prompt=prompt, zuzenex=run_zuzenex(s, prompt, batches, n_dec))
         elif model == "sakinex":

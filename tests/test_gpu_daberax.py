@@ -360,7 +360,7 @@ def test_delta_rule_rows_decode_rows_and_states():
     the stored state across calls cut anywhere, and a second sequence whose state stays untouched; states of 10 .. 500 rows."""
     check, stream, L, ptr = _api()
     g = torch.Generator().manual_seed(5)
-    for H, G, d, e in ((4, 2, 16, 16), (3, 3, 10, 6), (2, 1, 136, 40), (1, 1, 260, 33), (2, 2, 500, 8), (4, 1, 64, 300)):
+    for H, G, d, e in ((4, 2, 16, 16), (3, 3, 10, 6), (2, 1, 136, 40), (1, 1, 260, 33), (2, 2, 500, 8), (2, 2, 512, 8), (4, 1, 64, 300)):
         T = 45
         q, k, v, beta, dec = delta_inputs(g, T, H, G, d, e)
         rep = H // G
