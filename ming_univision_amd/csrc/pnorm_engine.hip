@@ -229,7 +229,9 @@ extern "C" int mn_pn_step(const mn_pn_model* m, const mn_pn_state* st, const flo
       MN_CHECK_LAUNCH("mn_pn_step(trace)");
     }
   }
-  MN_TRY(mn_axpy_rms_rows(xr, W, nullptr, W, 1.0f, m->final_w, m->eps, out, W, nullptr, 0, M, W, stream));
+  // decode rows: the one-workgroup-per-row launch with the row in registers (the other step functions' launch, here without a filter)
+  if (one_row && W <= 8192) MN_TRY(mn_axpy_rms_filter_rows(xr, W, nullptr, W, 1.0f, m->final_w, m->eps, nullptr, 0, nullptr, row_seq, row_slot, out, W, M, W, stream));
+  else MN_TRY(mn_axpy_rms_rows(xr, W, nullptr, W, 1.0f, m->final_w, m->eps, out, W, nullptr, 0, M, W, stream));
 #undef MN_TRY
   return MN_OK;
 }

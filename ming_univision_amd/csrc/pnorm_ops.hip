@@ -59,6 +59,37 @@ __global__ __launch_bounds__(256) void rms_scale_add_kernel(float* __restrict__ 
   }
 }
 
+// the same with the row in registers (rows of at most 256 VPT values): every load is issued before the reduction
+template <int VPT>
+__global__ __launch_bounds__(256) void rms_scale_add_reg_kernel(float* __restrict__ x, int64_t ldx, const float* __restrict__ y, int64_t ldy,
+                                                                const bf16_t* __restrict__ w, float eps, bf16_t* __restrict__ x16, int64_t ldx16,
+                                                                int n) {
+  __shared__ float red[4];
+  const int m = blockIdx.x, tid = threadIdx.x;
+  float yv[VPT], xv[VPT], wv[VPT];
+#pragma unroll
+  for (int t = 0; t < VPT; ++t) {
+    const int c = tid + 256 * t;
+    yv[t] = c < n ? y[(int64_t)m * ldy + c] : 0.f;
+    xv[t] = c < n ? x[(int64_t)m * ldx + c] : 0.f;
+    wv[t] = c < n ? bf16_to_f32(w[c]) : 0.f;
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int t = 0; t < VPT; ++t) ss = fmaf(yv[t], yv[t], ss);
+  ss = block_sum(ss, red);
+  const float den = sqrtf(ss / (float)n + eps);
+#pragma unroll
+  for (int t = 0; t < VPT; ++t) {
+    const int c = tid + 256 * t;
+    if (c < n) {
+      const float v = xv[t] + yv[t] / den * wv[t];
+      x[(int64_t)m * ldx + c] = v;
+      if (x16) x16[(int64_t)m * ldx16 + c] = f32_to_bf16(v);
+    }
+  }
+}
+
 __global__ __launch_bounds__(256) void gelu_mul_kernel(const float* __restrict__ a, int64_t lda, const float* __restrict__ b, int64_t ldb,
                                                        const bf16_t* __restrict__ table, int64_t ldt, const int32_t* __restrict__ idx,
                                                        float* __restrict__ y, int64_t ldy, bf16_t* __restrict__ y16, int64_t ldy16, int n) {
@@ -202,13 +233,14 @@ __device__ __forceinline__ float conv_silu(const DeltaPrepArgs& a, int m, int c,
   return silu_x(acc);
 }
 
+// grid (M, ceil(units / 4)): a wave takes one unit of a row — a q or k head (its unit norm is a wave's reduction) or 256 value channels
 __global__ __launch_bounds__(256) void delta_prep_kernel(DeltaPrepArgs a) {
-  const int m = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = blockIdx.x, tid = threadIdx.x, lane = tid & 63, unit = blockIdx.y * 4 + (tid >> 6);
   const int nqk = 2 * a.G * a.dim, nv = a.H * a.vdim, n = nqk + nv;
   const int seq = a.row_seq[m], slot = a.row_slot[m], back = a.row_back[m];
   float* out = a.qkv + (int64_t)m * a.ldo;
-  for (int j = wave; j < 2 * a.G; j += 4) {                       // one wave per q or k head
-    const int c0 = j * a.dim;
+  if (unit < 2 * a.G) {
+    const int c0 = unit * a.dim;
     float ss = 0.f;
     for (int d = lane; d < a.dim; d += 64) {
       const float v = conv_silu(a, m, c0 + d, n, seq, slot, back);
@@ -216,14 +248,18 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(DeltaPrepArgs a) {
       ss = fmaf(v, v, ss);
     }
     ss = wave_sum(ss);
-    const float r = (j < a.G ? a.q_scale : 1.0f) / sqrtf(ss + a.unit_eps);
+    const float r = (unit < a.G ? a.q_scale : 1.0f) / sqrtf(ss + a.unit_eps);
     for (int d = lane; d < a.dim; d += 64) out[c0 + d] *= r;      // the lane rereads what it wrote itself
+  } else {
+    const int e0 = (unit - 2 * a.G) * 256;
+    for (int e = e0 + lane; e < min(nv, e0 + 256); e += 64) out[nqk + e] = conv_silu(a, m, nqk + e, n, seq, slot, back);
   }
-  for (int e = tid; e < nv; e += 256) out[nqk + e] = conv_silu(a, m, nqk + e, n, seq, slot, back);
-  for (int h = tid; h < a.H; h += 256) {
-    const float* row = a.proj + (int64_t)m * a.ld;
-    a.bd[(int64_t)m * a.ldbd + h] = sigmoid_f(row[a.off_b + h]);
-    a.bd[(int64_t)m * a.ldbd + a.H + h] = expf(-expf(a.a_log[h]) * softplus_f(row[a.off_a + h] + a.dt_bias[h]));
+  if (blockIdx.y == 0) {
+    for (int h = tid; h < a.H; h += 256) {
+      const float* row = a.proj + (int64_t)m * a.ld;
+      a.bd[(int64_t)m * a.ldbd + h] = sigmoid_f(row[a.off_b + h]);
+      a.bd[(int64_t)m * a.ldbd + a.H + h] = expf(-expf(a.a_log[h]) * softplus_f(row[a.off_a + h] + a.dt_bias[h]));
+    }
   }
 }
 
@@ -554,7 +590,11 @@ __global__ __launch_bounds__(256) void head_rms_silu_gate_kernel(const float* __
 extern "C" int mn_rms_scale_add_rows(float* x, int64_t ldx, const float* y, int64_t ldy, const uint16_t* w, float eps, uint16_t* x16,
                                      int64_t ldx16, int M, int n, void* stream) {
   MN_CHECK_ARG(x && y && w && M >= 1 && n >= 1, "mn_rms_scale_add_rows: bad args");
-  hipLaunchKernelGGL(rms_scale_add_kernel, dim3((unsigned)M), dim3(256), 0, mn_stream(stream), x, ldx, y, ldy, w, eps, x16, ldx16, n);
+  hipStream_t st = mn_stream(stream);
+#define MN_RSA(V_) hipLaunchKernelGGL((rms_scale_add_reg_kernel<V_>), dim3((unsigned)M), dim3(256), 0, st, x, ldx, y, ldy, w, eps, x16, ldx16, n)
+  if (n <= 1024) MN_RSA(4); else if (n <= 2048) MN_RSA(8); else if (n <= 4096) MN_RSA(16); else if (n <= 8192) MN_RSA(32);
+  else hipLaunchKernelGGL(rms_scale_add_kernel, dim3((unsigned)M), dim3(256), 0, st, x, ldx, y, ldy, w, eps, x16, ldx16, n);
+#undef MN_RSA
   MN_CHECK_LAUNCH("mn_rms_scale_add_rows");
   return MN_OK;
 }
@@ -614,7 +654,9 @@ extern "C" int mn_delta_prep_rows(const float* proj, int64_t ld, int M, int H, i
                "mn_delta_prep_rows: bad args");
   DeltaPrepArgs a{proj, ld, H, G, dim, vdim, taps, off_b, off_a, w_conv, state, a_log, dt_bias, unit_eps, q_scale, row_seq, row_slot, row_back,
                   qkv, ldo, bd, ldbd};
-  hipLaunchKernelGGL(delta_prep_kernel, dim3((unsigned)M), dim3(256), 0, mn_stream(stream), a);
+  const int64_t units = 2 * (int64_t)G + mn_cdiv((int64_t)H * vdim, 256);
+  MN_CHECK_ARG(M <= 65535 * 32 && mn_cdiv(units, 4) <= 65535, "mn_delta_prep_rows: too many rows or channels");
+  hipLaunchKernelGGL(delta_prep_kernel, dim3((unsigned)M, (unsigned)mn_cdiv(units, 4)), dim3(256), 0, mn_stream(stream), a);
   MN_CHECK_LAUNCH("mn_delta_prep_rows");
   return MN_OK;
 }

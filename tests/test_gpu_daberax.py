@@ -155,7 +155,7 @@ def test_rotary_frequencies_in_all_three_bands():
 def test_result_norm_add_and_gelu_products():
     check, stream, L, ptr = _api()
     g = torch.Generator().manual_seed(0)
-    for M, n in ((5, 44), (3, 1), (70, 1000)):
+    for M, n in ((5, 44), (3, 1), (70, 1000), (2, 2100), (3, 8200)):
         x, y, w = torch.randn(M, n + 3, generator=g), 4 * torch.randn(M, n + 1, generator=g), _bf(1 + 0.2 * torch.randn(n, generator=g))
         xd, x16 = x.cuda(), torch.zeros(M, n, dtype=torch.bfloat16, device="cuda")
         check(L.mn_rms_scale_add_rows(ptr(xd), n + 3, ptr(D(y)), n + 1, ptr(D(w)), 1e-3, ptr(x16), n, M, n, stream()))
