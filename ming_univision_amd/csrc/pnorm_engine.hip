@@ -186,6 +186,7 @@ extern "C" int mn_pn_step(const mn_pn_model* m, const mn_pn_state* st, const flo
       if (l.window > 0 && l.window + 3 < keys) keys = l.window + 3;
       // latent attention's decode rows run on the matrix-core kernel (all heads of a row in one workgroup): its key tiles hold 16 keys
       int ns = mn_window_attn_splits_tile(n_blk, H, G, one_row, keys, latent && one_row ? 16 : 64);
+      if (latent && one_row && (int64_t)ns * d.avd > 16384) ns = 16384 / d.avd > 1 ? 16384 / d.avd : 1;   // the merge reads ns x 16 x avd partial sums a row
       while (ns > 1 && mn_window_attn_workspace_bytes(n_blk, H, G, d.avd, one_row, ns) > p.attn_ws) --ns;
       const bool gate = attn && l.has_gate;
       MN_TRY(mn_window_pool_attn_blocks_cap(qf, d.nq, karena, ldk, varena, ldv, nullptr, nullptr, nullptr, l.softcap, row_seq, row_slot, blk_tab,
