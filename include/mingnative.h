@@ -91,7 +91,8 @@ enum mn_epilogue {
   MN_EPI_GELU = 2,        /* exact erf GELU (nn.GELU default) */
   MN_EPI_SWIGLU = 3,      /* out[n] = silu(y[n]) * y[n + N]; W and bias hold 2N rows (chunk(2), swiglu_ffn.py:30-34) */
   MN_EPI_RESID = 4,       /* out = res + y */
-  MN_EPI_RESID_GATE = 5   /* out = res + gate * y   (ResBlock, diff_loss_rf_swiglu.py:272) */
+  MN_EPI_RESID_GATE = 5,  /* out = res + gate * y   (ResBlock, diff_loss_rf_swiglu.py:272) */
+  MN_EPI_GEGLU_TANH = 6   /* out[n] = gelu_tanh(y[n]) * y[n + N], gelu in its tanh form; W and bias hold 2N rows like MN_EPI_SWIGLU (bf16 weights only) */
 };
 
 typedef struct mn_skinny_args {

@@ -92,6 +92,9 @@ __device__ __forceinline__ mn_u4_t fp8x8_to_bf16(uint32_t q0, uint32_t q1) {
 // ---- activations ----------------------------------------------------------------------------
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
 __device__ __forceinline__ float gelu_erf_f(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
+__device__ __forceinline__ float gelu_tanh_f(float z) { return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
+// epilogues whose weights hold two row sets per output (the second set at row n + N)
+static inline bool mn_epi_pairs(int epilogue) { return epilogue == MN_EPI_SWIGLU || epilogue == MN_EPI_GEGLU_TANH; }
 
 // ---- wave / block reductions -------------------------------------------------------------
 // Cross-lane reductions on DPP operands: `__shfl_xor` compiles to ds_bpermute_b32 here — one trip through the LDS crossbar per step

@@ -211,8 +211,12 @@ extern "C" int mn_pn_step(const mn_pn_model* m, const mn_pn_state* st, const flo
     MN_TRY(mn_rms_scale_add_rows(xr, W, yf, W, l.norm1, m->eps, xh, W, M, W, stream));
     // ---- feed-forward ----
     if (l.ff > 0) {
-      MN_TRY(linear(arith, M, xr, W, xh, W, l.w_gate_up, 2 * l.ff, W, nullptr, gu, 2 * l.ff, gws, gwb, stream));
-      MN_TRY(mn_gelu_mul_rows(gu, 2 * l.ff, gu + l.ff, 2 * l.ff, nullptr, 0, nullptr, act, l.ff, acth, l.ff, M, l.ff, stream));
+      bool fused = false;                                // few rows: the gelu product rides the weight-streaming product's epilogue
+      if (!acth) MN_TRY(linear_geglu(arith, M, xr, W, l.w_gate_up, l.ff, W, act, l.ff, gws, gwb, stream, &fused));
+      if (!fused) {
+        MN_TRY(linear(arith, M, xr, W, xh, W, l.w_gate_up, 2 * l.ff, W, nullptr, gu, 2 * l.ff, gws, gwb, stream));
+        MN_TRY(mn_gelu_mul_rows(gu, 2 * l.ff, gu + l.ff, 2 * l.ff, nullptr, 0, nullptr, act, l.ff, acth, l.ff, M, l.ff, stream));
+      }
       MN_TRY(linear(arith, M, act, l.ff, acth, l.ff, l.w_down, W, l.ff, nullptr, yf, W, gws, gwb, stream));
       MN_TRY(mn_rms_scale_add_rows(xr, W, yf, W, l.norm2, m->eps, xh, W, M, W, stream));
     }

@@ -34,6 +34,23 @@ inline int linear(int arith, int M, const float* A, int64_t lda, const uint16_t*
   return mn_gemm_f32_batched(A, lda, 0, W, K, 0, bias, C, ldc, 0, nullptr, 0, 0, nullptr, 0, 0, M, N, K, 1, 1.0f, stream);
 }
 
+// act fp32 [M, N] = gelu_tanh(A Wg^T) * (A Wu^T) with W = [Wg ; Wu] (2N rows) as the EPILOGUE of the weight-streaming product, for steps
+// that take that route (<= 8 rows, or 9 .. 64 rows with scratch in the bf16 arithmetic).  *done says whether the step
+// took it; if not, the caller runs the plain product and the activation launch.
+inline int linear_geglu(int arith, int M, const float* A, int64_t lda, const uint16_t* W, int N, int K, float* act, int64_t ldact, void* gws,
+                        size_t gws_bytes, void* stream, bool* done) {
+  *done = false;
+  const bool stream_mfma = arith == MN_SEQ_ARITH_BF16 && M > 8 && M <= 64 && gws && gws_bytes >= mn_skinny_workspace_bytes(M, N, K, MN_EPI_GEGLU_TANH);
+  if (!((M <= 8 || stream_mfma) && mfma_ok(W, K))) return MN_OK;
+  mn_skinny_args a;
+  memset(&a, 0, sizeof(a));
+  a.x = A; a.ldx = lda; a.w = W; a.ldw = K; a.out = act; a.ldo = ldact;
+  a.M = M; a.N = N; a.K = K; a.epilogue = MN_EPI_GEGLU_TANH;
+  if (M > 8) { a.ws = gws; a.ws_bytes = gws_bytes; }
+  *done = true;
+  return mn_skinny_gemm(&a, stream);
+}
+
 // the step's own copy of its input rows (a kernel, not a memcpy node: the step may be captured into a graph)
 __global__ void copy_rows_kernel(const float* __restrict__ x, int64_t ldx, float* __restrict__ y, int n) {
   const int c = blockIdx.x * 256 + threadIdx.x;

@@ -152,6 +152,11 @@ __global__ __launch_bounds__(NT) void skinny_kernel(const KArgs ka) {
                 if (a.bias) y2 += bf16_to_f32(a.bias[n + N]);
                 y = silu_f(y) * y2;
               } break;
+              case MN_EPI_GEGLU_TANH: {
+                float y2 = acc[SW - 1][r][m];
+                if (a.bias) y2 += bf16_to_f32(a.bias[n + N]);
+                y = gelu_tanh_f(y) * y2;
+              } break;
               case MN_EPI_RESID:
                 y += a.res[(int64_t)b * a.res_batch_stride + (int64_t)m * a.ldres + n];
                 break;
@@ -282,6 +287,11 @@ __global__ __launch_bounds__(256) void medium_epilogue_kernel(const mn_skinny_ar
       if (a.bias) y2 += bf16_to_f32(a.bias[n + N]);
       y = silu_f(y) * y2;
     } break;
+    case MN_EPI_GEGLU_TANH: {
+      float y2 = gather(n + N);
+      if (a.bias) y2 += bf16_to_f32(a.bias[n + N]);
+      y = gelu_tanh_f(y) * y2;
+    } break;
     case MN_EPI_RESID: y += a.res[(int64_t)m * a.ldres + n]; break;
     case MN_EPI_RESID_GATE: y = a.res[(int64_t)m * a.ldres + n] + a.gate[(int64_t)m * a.ldgate + n] * y; break;
     default: break;
@@ -307,7 +317,7 @@ constexpr int MEDIUM_MIN_M = 2;
 
 extern "C" size_t mn_skinny_workspace_bytes(int M, int N, int K, int epilogue) {
   if (M < MEDIUM_MIN_M) return 0;
-  const int Ntot = epilogue == MN_EPI_SWIGLU ? 2 * N : N;
+  const int Ntot = mn_epi_pairs(epilogue) ? 2 * N : N;
   const size_t y = ((size_t)2 * M * K * sizeof(bf16_t) + 255) & ~(size_t)255;
   return y + (size_t)mn_stream_mfma_slices(M, Ntot, K) * M * Ntot * sizeof(float) + 256;
 }
@@ -315,7 +325,7 @@ extern "C" size_t mn_skinny_workspace_bytes(int M, int N, int K, int epilogue) {
 // quantised weights (wfmt != 0): every row count takes the matrix-core route (the fp32-FMA kernel reads bf16 rows)
 extern "C" size_t mn_skinny_workspace_bytes_wq(int wfmt, int M, int N, int K, int epilogue) {
   if (wfmt == MN_W_BF16) return mn_skinny_workspace_bytes(M, N, K, epilogue);
-  const int Ntot = epilogue == MN_EPI_SWIGLU ? 2 * N : N;
+  const int Ntot = mn_epi_pairs(epilogue) ? 2 * N : N;
   const size_t y = ((size_t)2 * M * K * sizeof(bf16_t) + 255) & ~(size_t)255;
   return y + (size_t)mn_stream_mfma_wq_slices(wfmt, M, Ntot, K) * M * Ntot * sizeof(float) + 256;
 }
@@ -327,7 +337,7 @@ static int skinny_medium(const mn_skinny_args& a, void* stream) {
   MN_CHECK_ARG(a.M <= 64, "mn_skinny_gemm: M=%d out of range [1,64]", a.M);
   MN_CHECK_ARG((a.batch <= 1) && (a.nseg <= 1), "mn_skinny_gemm: batch/nseg forms need M <= 8");
   MN_CHECK_ARG(a.ldw == a.K, "mn_skinny_gemm: M > 8 needs densely packed weights (ldw == K)");
-  const int Ntot = a.epilogue == MN_EPI_SWIGLU ? 2 * a.N : a.N;
+  const int Ntot = mn_epi_pairs(a.epilogue) ? 2 * a.N : a.N;
   const bool w8 = a.wfmt != MN_W_BF16;
   MN_CHECK_ARG(!w8 || (a.wscale && (a.K % 16) == 0), "mn_skinny_gemm: fp8 weights need wscale and K %% 16 == 0");
   MN_CHECK_ARG(a.wfmt != MN_W_NF4 || (a.K % 64) == 0, "mn_skinny_gemm: NF4 weights need K %% 64 == 0");
@@ -361,7 +371,8 @@ extern "C" int mn_skinny_gemm(const mn_skinny_args* args, void* stream) {
   MN_CHECK_ARG((a.ldw % 8) == 0, "mn_skinny_gemm: ldw=%lld must be a multiple of 8", (long long)a.ldw);
   MN_CHECK_ARG(a.x && a.w && a.out, "mn_skinny_gemm: null pointer");
   MN_CHECK_ARG(a.prologue >= 0 && a.prologue <= MN_PRO_LN_MOD, "mn_skinny_gemm: bad prologue %d", a.prologue);
-  MN_CHECK_ARG(a.epilogue >= 0 && a.epilogue <= MN_EPI_RESID_GATE, "mn_skinny_gemm: bad epilogue %d", a.epilogue);
+  MN_CHECK_ARG(a.epilogue >= 0 && a.epilogue <= MN_EPI_GEGLU_TANH, "mn_skinny_gemm: bad epilogue %d", a.epilogue);
+  MN_CHECK_ARG(a.epilogue != MN_EPI_GEGLU_TANH || a.wfmt == MN_W_BF16, "mn_skinny_gemm: the gelu product epilogue takes bf16 weights");
   ka.nseg = a.nseg > 0 ? a.nseg : 1;
   ka.batch = a.batch > 0 ? a.batch : 1;
   MN_CHECK_ARG(a.wfmt == MN_W_BF16 || a.wfmt == MN_W_FP8_E4M3 || a.wfmt == MN_W_INT8 || a.wfmt == MN_W_NF4, "mn_skinny_gemm: bad wfmt %d", a.wfmt);
@@ -411,7 +422,7 @@ extern "C" int mn_skinny_gemm(const mn_skinny_args* args, void* stream) {
     return MN_OK;
   }
 
-  const int sw = a.epilogue == MN_EPI_SWIGLU ? 2 : 1;
+  const int sw = mn_epi_pairs(a.epilogue) ? 2 : 1;
   // Occupancy plan: ~16 waves per CU (each keeps RING x SW x R KiB of weights in flight), blocks per CU
   // limited by the LDS image of x; a wave should own >= 2 row groups where N allows so that the
   // per-block prologue is amortised and the next group's loads overlap the current reduction.

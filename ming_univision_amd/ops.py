@@ -12,7 +12,7 @@ from . import _lib
 from ._lib import SkinnyArgs, check, current_stream, lib, ptr
 
 PRO = dict(none=0, silu=1, add_silu=2, rmsnorm=3, ln=4, ln_mod=5)
-EPI = dict(none=0, silu=1, gelu=2, swiglu=3, resid=4, resid_gate=5)
+EPI = dict(none=0, silu=1, gelu=2, swiglu=3, resid=4, resid_gate=5, geglu_tanh=6)
 GEMM_EPI = dict(bf16=0, bf16_gelu=1, f32=2, f32_resid=3)
 
 
@@ -41,7 +41,7 @@ def skinny_gemm(x, w, bias=None, *, prologue="none", epilogue="none", out=None, 
     _req(pro_a, torch.float32, "pro_a"); _req(pro_b, torch.float32, "pro_b")
     _req(res, torch.float32, "res"); _req(gate, torch.float32, "gate")
     M, K = x.shape
-    N = w.shape[0] // 2 if epilogue == "swiglu" else w.shape[0]
+    N = w.shape[0] // 2 if epilogue in ("swiglu", "geglu_tanh") else w.shape[0]
     if n_out is not None:
         N = n_out
     assert w.shape[1] == (K // 2 if (wscale is not None and wfmt == "int4") else K) and x.stride(1) == 1 and w.stride(1) == 1

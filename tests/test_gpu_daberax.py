@@ -459,6 +459,20 @@ def test_head_gates():
         assert err(xd, ref) < 1e-6 and err(y16.float(), ref) < 1e-2
 
 
+def test_gelu_product_as_the_streaming_products_epilogue():
+    """gelu(x Wg^T) * (x Wu^T) in the epilogue of the weight-streaming product, on its fp32 FMA kernels (1 .. 8 rows) and its matrix-core
+    route (more rows, hi/lo operands), against the plain product followed by the activation."""
+    from ming_univision_amd import ops
+    g = torch.Generator().manual_seed(10)
+    for M, N, K in ((1, 40, 64), (3, 320, 200), (8, 96, 2048), (20, 64, 256), (64, 136, 512)):
+        x = torch.randn(M, K, generator=g)
+        w = _bf(torch.randn(2 * N, K, generator=g) * K ** -0.5)
+        got = ops.skinny_gemm(x.cuda(), w.cuda(), epilogue="geglu_tanh")
+        y = x.double() @ w.double().T
+        ref = O.gelu_tanh(y[:, :N]) * y[:, N:]
+        assert got.shape == (M, N) and err(got, ref) < (1e-5 if M <= 8 else 2e-4), (M, N, K)
+
+
 # ---- whole models ------------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("name", MODELS)
 def test_prompt_layers_and_logits(name):
