@@ -328,8 +328,8 @@ def daberax_config(s, window=1024):
     from .configuration import DaberaxConfig
     H = s["heads"]
     mlp = dict(kind="dense", ff=s["ff"])
-    att = dict(type="attention", mixer=dict(heads=H, kv_heads=H // 4, dim=128, vdim=128, scale=128 ** -0.5, softcap=30.0, mask=dict(size=window),
-                                            rot=dict(base=500000.0, dims=128, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))), mlp=mlp)
+    att = dict(type="attention", mixer=dict(heads=H, kv_heads=H // 4, dim=128, vdim=128, scale=128 ** -0.5, softcap=50.0, mask=dict(size=window),
+                                            rot=dict(base=1000000.0, dims=128, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))), mlp=mlp)
     lat = dict(type="latent_attention", mixer=dict(heads=H, dim=128, rot_dim=64, vdim=128, kv_rank=s["kv_rank"], scale=192 ** -0.5,
                                                    mask=dict(size=window), rot=dict(base=10000.0, dims=64)), mlp=mlp)
     dlt = dict(type="delta", mixer=dict(heads=H, kv_heads=H // 2, dim=128, vdim=128, conv=4), mlp=mlp)
@@ -392,7 +392,7 @@ def run_daberax(s, T, batches, n_dec, window=1024):
         def attn(M, rs, rp, one_row):
             n_blk = M if one_row else tabs["blk_tab"].shape[0]
             ns = lib().mn_window_attn_splits_tile(n_blk, H, G, one_row, seen, 16 if (v_of_k and one_row) else 64)
-            check(lib().mn_window_pool_attn_blocks_cap(ptr(q), H * dk, ptr(st["k"]), ldk, ptr(varena), ldk if v_of_k else 0, None, None, None, 30.0,
+            check(lib().mn_window_pool_attn_blocks_cap(ptr(q), H * dk, ptr(st["k"]), ldk, ptr(varena), ldk if v_of_k else 0, None, None, None, 50.0,
                                                        ptr(rs), ptr(rp), None if one_row else ptr(tabs["blk_tab"]), n_blk, one_row, H, G, dk, dv,
                                                        dec.t_max, 1, window, 0, 1.0, ptr(att), H * dv, None, 0, ns, ptr(aws), aws.numel(), -1,
                                                        current_stream()), "mn_window_pool_attn_blocks_cap")

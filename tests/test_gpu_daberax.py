@@ -142,12 +142,12 @@ def dev_freq(rot):
 
 # ---- operators alone -------------------------------------------------------------------------------------------------------
 def test_rotary_frequencies_in_all_three_bands():
-    for rot in ({"base": 10000.0, "dims": 64}, {"base": 500000.0, "dims": 48, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 256}},
+    for rot in ({"base": 10000.0, "dims": 64}, {"base": 300000.0, "dims": 40, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 256}},
                 {"base": 100.0, "dims": 6, "scaling": {"factor": 3.0, "low": 0.5, "high": 2.5, "original": 40}}):
         got, ref = dev_freq(rot).cpu().double(), O.rotary_frequencies(rot)
         assert float(((got - ref) / ref).abs().max()) < 1e-7
-    sc = {"base": 500000.0, "dims": 48, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 256}}
-    plain = O.rotary_frequencies({"base": 500000.0, "dims": 48})
+    sc = {"base": 300000.0, "dims": 40, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 256}}
+    plain = O.rotary_frequencies({"base": 300000.0, "dims": 40})
     ratio = O.rotary_frequencies(sc) / plain
     assert float(ratio[0]) == 1.0 and abs(float(ratio[-1]) - 1 / 8.0) < 1e-12 and bool(((ratio > 0.126) & (ratio < 0.999)).any())
 
@@ -179,7 +179,7 @@ def test_whole_projection_norms_rotation_and_append():
     check, stream, L, ptr = _api()
     g = torch.Generator().manual_seed(1)
     for H, G, d, e, rot in ((4, 2, 16, 16, {"base": 1e4, "dims": 16}), (3, 1, 10, 18, {"base": 500.0, "dims": 6}), (1, 1, 130, 5, None),
-                            (5, 5, 64, 72, {"base": 5e5, "dims": 64, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 128}})):
+                            (5, 5, 64, 72, {"base": 2e5, "dims": 64, "scaling": {"factor": 6.0, "low": 1.0, "high": 3.0, "original": 128}})):
         spans = [(1, 7, 0), (0, 1, 2999), (2, 5, 94)]
         M, t_max, n_seq, eps, scale = 13, 3004, 3, 1e-5, 0.37
         r = _rows(spans)
@@ -252,7 +252,7 @@ def test_attention_needles_at_window_tile_and_split_edges(variant):
     """One key decides a row: the first slot, the row's own slot, the oldest slot inside the window (it must be seen) and the one
     before it (it must not), across 16- and 64-key tile edges and forced key splits, in runs of rows of a prompt."""
     for H, G, d, e in ((4, 2, 16, 16), (3, 1, 10, 18), (2, 2, 72, 136)):
-        for window, cap in ((0, 0.0), (40, 0.0), (136, 30.0), (17, 5.0), (1, 0.0)):
+        for window, cap in ((0, 0.0), (24, 0.0), (120, 25.0), (17, 5.0), (1, 0.0)):
             T = 300
             rows = [200, 201, 202, 203, 204, 205]                   # two runs: four rows and two rows
             lo = lambda p: max(0, p - window + 1) if window else 0  # noqa: E731
@@ -270,7 +270,7 @@ def test_attention_needles_at_window_tile_and_split_edges(variant):
 def test_attention_needles_in_decode_rows():
     """The same for rows that are alone in the step (the decode form: key splits and their merge)."""
     for H, G, d, e in ((4, 2, 16, 16), (12, 1, 8, 8), (3, 3, 130, 260)):
-        for window, cap in ((0, 0.0), (40, 0.0), (136, 30.0), (17, 0.0)):
+        for window, cap in ((0, 0.0), (24, 0.0), (120, 25.0), (17, 0.0)):
             T = 700
             p = 650
             lo = max(0, p - window + 1) if window else 0
