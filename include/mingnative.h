@@ -1206,10 +1206,11 @@ MN_API int mn_head_sigmoid_gate_rows(float* x, int64_t ldx, const float* g, int6
 /* Gated delta rule, preparation.  proj fp32 [M, ld]: raw channels [q: G dim ; k: G dim ; v: H vdim] from column 0, the write-strength
  * logits [H] from off_b and the decay logits [H] from off_a.  Every channel goes through its causal filter w_conv bf16 [channels, taps]
  * (last tap = the current row; earlier inputs from the rows before it in this call, then from state fp32 [n_seq, taps - 1, channels]
- * as mn_tap_filter_rows reads it — mn_tap_state_update moves it on afterwards) and silu; q and k heads become x / sqrt(sum(x^2) +
- * unit_eps), q also times q_scale.  qkv fp32 [M, channels]; bd fp32 [M, 2 H] = [sigmoid(b) ; exp(-exp(a_log) softplus(a + dt_bias))]. */
+ * as mn_tap_filter_rows reads it) and silu; q and k heads become x / sqrt(sum(x^2) + unit_eps), q also times q_scale.  advance_state 0:
+ * the state is read only and mn_tap_state_update moves it on afterwards; 1 (every row alone in its sequence, a decode step): the
+ * launch moves it on by this row itself.  qkv fp32 [M, channels]; bd fp32 [M, 2 H] = [sigmoid(b) ; exp(-exp(a_log) softplus(a + dt_bias))]. */
 MN_API int mn_delta_prep_rows(const float* proj, int64_t ld, int M, int H, int G, int dim, int vdim, int off_b, int off_a,
-                              const uint16_t* w_conv, int taps, const float* state, const float* a_log, const float* dt_bias,
+                              const uint16_t* w_conv, int taps, float* state, int advance_state, const float* a_log, const float* dt_bias,
                               float unit_eps, float q_scale, const int32_t* row_seq, const int32_t* row_slot, const int32_t* row_back,
                               float* qkv, int64_t ldo, float* bd, int64_t ldbd, void* stream);
 /* Gated delta rule over each sequence's rows, per head h (q / k head h / (H / G)) with beta and g of the row:

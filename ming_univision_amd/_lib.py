@@ -401,7 +401,7 @@ SYMBOLS = {
     "mn_proj_norm_rope_append": (_i, [_p, _i64, _i, _i, _i, _i, _i, _p, _p, _f, _i, _i, _p, _f, _p, _p, _p, _i64, _p, _i64, _p, _i64, _i, _p]),
     "mn_latent_rope_append": (_i, [_p, _i64, _i, _i, _i, _i, _i, _p, _f, _i, _i, _p, _f, _p, _p, _p, _i64, _p, _i64, _i, _p]),
     "mn_head_sigmoid_gate_rows": (_i, [_p, _i64, _p, _i64, _p, _i64, _i, _i, _i, _p]),
-    "mn_delta_prep_rows": (_i, [_p, _i64, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p, _f, _f, _p, _p, _p, _p, _i64, _p, _i64, _p]),
+    "mn_delta_prep_rows": (_i, [_p, _i64, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _i, _p, _p, _f, _f, _p, _p, _p, _p, _i64, _p, _i64, _p]),
     "mn_gated_delta_rows": (_i, [_p, _i64, _p, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _p, _i, _p, _i64, _p]),
     "mn_head_rms_silu_gate_rows": (_i, [_p, _i64, _p, _f, _p, _i64, _p, _i64, _p, _i64, _i, _i, _i, _p]),
     "mn_pn_workspace_bytes": (_sz, [C.POINTER(PnModel), _i]),

@@ -198,10 +198,11 @@ extern "C" int mn_pn_step(const mn_pn_model* m, const mn_pn_state* st, const flo
                                    l.vdim, nullptr, 0, 0, M, l.vdim, l.kv_rank, H, 1.0f, stream));
     } else {
       const int chan = d.nq;
-      MN_TRY(mn_delta_prep_rows(pin, d.n_in, M, l.heads, l.kv_heads, l.dim, l.vdim, d.off_b, d.off_a, l.w_conv, l.conv, st->conv[li], l.a_log,
-                                l.dt_bias, l.unit_eps, 1.0f / sqrtf((float)l.dim), row_seq, row_slot, row_back, qf, chan, bd, 2 * l.heads,
-                                stream));
-      if (l.conv > 1) MN_TRY(mn_tap_state_update(pin, d.n_in, l.conv, st->conv[li], row_seq, row_back, M, chan, stream));
+      // decode rows move their filter state on inside the preparation launch
+      MN_TRY(mn_delta_prep_rows(pin, d.n_in, M, l.heads, l.kv_heads, l.dim, l.vdim, d.off_b, d.off_a, l.w_conv, l.conv, st->conv[li], one_row ? 1 : 0,
+                                l.a_log, l.dt_bias, l.unit_eps, 1.0f / sqrtf((float)l.dim), row_seq, row_slot, row_back, qf, chan, bd,
+                                2 * l.heads, stream));
+      if (l.conv > 1 && !one_row) MN_TRY(mn_tap_state_update(pin, d.n_in, l.conv, st->conv[li], row_seq, row_back, M, chan, stream));
       MN_TRY(mn_gated_delta_rows(qf, chan, bd, 2 * l.heads, M, l.heads, l.kv_heads, l.dim, l.vdim, st->lin[li], row_seq, row_slot, row_back,
                                  one_row ? MN_SEQ_ROWS_DISTINCT : 0, mid, d.nmid, stream));
       MN_TRY(mn_head_rms_silu_gate_rows(mid, d.nmid, l.mix_norm, m->eps, pin + d.off_g, d.n_in, cat, d.hv, cath, d.hv, M, l.heads, l.vdim,

@@ -211,7 +211,8 @@ struct DeltaPrepArgs {
   const float* proj; int64_t ld;             // raw [q ; k ; v] at column 0, b at off_b, a at off_a
   int H, G, dim, vdim, taps, off_b, off_a;
   const bf16_t* w_conv;                      // [2 G dim + H vdim, taps], the last tap multiplies the current row
-  const float* state;                        // [n_seq, taps - 1, channels]
+  float* state;                              // [n_seq, taps - 1, channels]
+  int advance;                               // 1: every row is alone in its sequence and moves the state on by itself
   const float *a_log, *dt_bias;              // device fp32 [H]
   float unit_eps, q_scale;
   const int32_t *row_seq, *row_slot, *row_back;
@@ -226,6 +227,11 @@ __device__ __forceinline__ float conv_silu(const DeltaPrepArgs& a, int m, int c,
     if (k <= back) v = a.proj[(int64_t)(m - k) * a.ld + c];
     else if (slot - k >= 0) v = a.state[((int64_t)seq * (a.taps - 1) + (k - back - 1)) * n + c];
     acc = fmaf(bf16_to_f32(a.w_conv[(int64_t)c * a.taps + (a.taps - 1 - k)]), v, acc);
+  }
+  if (a.advance && a.taps > 1) {                // a one-row sequence: entry i becomes entry i - 1, entry 0 this row's input
+    float* st = a.state + (int64_t)seq * (a.taps - 1) * n + c;
+    for (int i = a.taps - 2; i >= 1; --i) st[(int64_t)i * n] = st[(int64_t)(i - 1) * n];
+    st[0] = a.proj[(int64_t)m * a.ld + c];
   }
   return silu_x(acc);
 }
@@ -643,13 +649,13 @@ extern "C" int mn_head_sigmoid_gate_rows(float* x, int64_t ldx, const float* g, 
 }
 
 extern "C" int mn_delta_prep_rows(const float* proj, int64_t ld, int M, int H, int G, int dim, int vdim, int off_b, int off_a,
-                                  const uint16_t* w_conv, int taps, const float* state, const float* a_log, const float* dt_bias,
-                                  float unit_eps, float q_scale, const int32_t* row_seq, const int32_t* row_slot, const int32_t* row_back,
-                                  float* qkv, int64_t ldo, float* bd, int64_t ldbd, void* stream) {
+                                  const uint16_t* w_conv, int taps, float* state, int advance_state, const float* a_log,
+                                  const float* dt_bias, float unit_eps, float q_scale, const int32_t* row_seq, const int32_t* row_slot,
+                                  const int32_t* row_back, float* qkv, int64_t ldo, float* bd, int64_t ldbd, void* stream) {
   MN_CHECK_ARG(proj && w_conv && a_log && dt_bias && row_seq && row_slot && row_back && qkv && bd && M >= 1 && H >= 1 && G >= 1 && (H % G) == 0 &&
                    dim >= 1 && vdim >= 1 && taps >= 1 && (taps == 1 || state) && ldbd >= 2 * (int64_t)H,
                "mn_delta_prep_rows: bad args");
-  DeltaPrepArgs a{proj, ld, H, G, dim, vdim, taps, off_b, off_a, w_conv, state, a_log, dt_bias, unit_eps, q_scale, row_seq, row_slot, row_back,
+  DeltaPrepArgs a{proj, ld, H, G, dim, vdim, taps, off_b, off_a, w_conv, state, advance_state ? 1 : 0, a_log, dt_bias, unit_eps, q_scale, row_seq, row_slot, row_back,
                   qkv, ldo, bd, ldbd};
   const int64_t units = 2 * (int64_t)G + mn_cdiv((int64_t)H * vdim, 256);
   MN_CHECK_ARG(M <= 65535 * 32 && mn_cdiv(units, 4) <= 65535, "mn_delta_prep_rows: too many rows or channels");
